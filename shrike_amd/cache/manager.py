@@ -22,7 +22,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
-from ..parts.base import PagedSpec, StateSpec
+from ..parts.base import CompositeSpec, PagedSpec, StateSpec
 from .pages import PageError, PagePool, SlotPool
 
 
@@ -52,6 +52,8 @@ class LayerCache:
     # a fixed-size (graph) batch carry the slot index `slots`, which only this
     # view holds, so whatever they write disturbs no request
     state_padded: object = None
+    # for a mixer made of several mixers: sub-name -> the LayerCache of each that keeps something
+    parts: dict = field(default_factory=dict)
 
 
 class PageGroup:
@@ -86,10 +88,10 @@ class CacheManager:
         self.num_pages = num_pages
         self.groups: list[PageGroup] = []
         self.state_groups: list[StateGroup] = []
-        self._where: dict[int, tuple[str, int, int]] = {}  # position -> (family, group, index)
-        for pos, spec in enumerate(layer_specs):
-            if spec is None:
-                continue
+        # position -> (family, group, index), or for a composite need {sub-name: that triple}
+        self._where: dict[int, object] = {}
+
+        def place(pos: int, spec) -> tuple[str, int, int]:
             if isinstance(spec, PagedSpec):
                 family, groups, make = "pages", self.groups, lambda s: PageGroup(s, num_pages)
             elif isinstance(spec, StateSpec):
@@ -102,8 +104,16 @@ class CacheManager:
             else:
                 groups.append(make(spec))
                 gi = len(groups) - 1
-            self._where[pos] = (family, gi, len(groups[gi].layers))
             groups[gi].layers.append(pos)
+            return family, gi, len(groups[gi].layers) - 1
+
+        for pos, spec in enumerate(layer_specs):
+            if spec is None:
+                continue
+            if isinstance(spec, CompositeSpec):
+                self._where[pos] = {name: place(pos, sub) for name, sub in spec.parts}
+            else:
+                self._where[pos] = place(pos, spec)
         self.slots = SlotPool(max_slots)
         # A prefix can only be shared where every layer's cache is a pure
         # function of the prefix, page by page: no window, no state.
@@ -150,7 +160,14 @@ class CacheManager:
     def layer_cache(self, position: int, reader: bool = False) -> LayerCache:
         """The cache of schedule position `position`; `reader` marks a layer that
         only reads it."""
-        family, gi, li = self._where[position]
+        where = self._where[position]
+        if isinstance(where, dict):
+            return LayerCache(group=-1, owned=not reader, page_size=self.page_size,
+                              parts={name: self._one_cache(w, reader) for name, w in where.items()})
+        return self._one_cache(where, reader)
+
+    def _one_cache(self, where: tuple, reader: bool) -> LayerCache:
+        family, gi, li = where
         if family == "pages":
             g = self.groups[gi]
             return LayerCache(

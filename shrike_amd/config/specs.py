@@ -31,6 +31,17 @@ class RMSNormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * weight + bias, var the mean of the squared
+    deviations; ``bias`` False: no bias tensor."""
+
+    kind: ClassVar[str] = "layernorm"
+    eps: float
+    bias: bool = True
+    names: Names = ()
+
+
+@dataclass(frozen=True)
 class RotarySpec:
     """Rotation of element pairs (i, i + rotary_dim/2) by position * theta**(-2i/rotary_dim)."""
 
@@ -67,6 +78,11 @@ class AttentionSpec:
     (coef, every): the queries at position p are multiplied by 1 + coef *
     ln(floor((p + 1) / every) + 1).  ``value_norm_eps``: each head's value is divided
     by sqrt(mean(v^2) + eps), without a weight, before it is cached.
+    ``distance_bias``: two learned numbers per query head (r1, r2); r1 * ln(1 + r2 * (i - j))
+    is taken off the scaled score of query i and key j.  ``fixed_sink``: a sink of this fixed
+    score (no tensor) in every head's denominator.  ``talking_heads``: a learned [heads, heads]
+    matrix T mixes the softmax weights across heads, w_h = sum_g T[h, g] p_g, before head h
+    applies them to the values of its own key/value head (the sink's share is not mixed).
     """
 
     kind: ClassVar[str] = "paged_attention"
@@ -86,6 +102,9 @@ class AttentionSpec:
     sinks: bool = False
     query_temperature: tuple | None = None
     value_norm_eps: float | None = None
+    distance_bias: bool = False
+    fixed_sink: float | None = None
+    talking_heads: bool = False
 
 
 @dataclass(frozen=True)
@@ -136,6 +155,75 @@ class MLSTMSpec:
     value_dim: int
     gate_cap: float
     eps: float
+    names: Names = ()
+
+
+@dataclass(frozen=True)
+class SelectiveScanSpec:
+    """The selective scan of Mamba.  W_in x is [u: inner | z: inner]; u passes a causal
+    convolution per channel (``conv`` taps, the last meets the current token, with a bias) and
+    SiLU; W_x u is [dt: dt_rank | B: state | C: state]; dt <- softplus(W_dt dt + b) per channel;
+    A = -exp(A_log) [inner, state];  S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c u_c B_n;
+    y_c = sum_n S[c, n] C_n + D_c u_c;  out = W_o (y * silu(z)).  Per request: S (float32) and
+    the convolution's last conv - 1 inputs."""
+
+    kind: ClassVar[str] = "selective_scan"
+    inner: int
+    state: int
+    dt_rank: int
+    conv: int
+    names: Names = ()
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head, no softmax and no denominator.  q = W_q x,
+    k = W_k x ([heads, head_dim]), v = W_v x ([heads, value_dim]); ``position`` (a rotation
+    spec or None) is applied to q and k; k is multiplied by head_dim ** -0.5;
+    S_t = decay[h] S_(t-1) + k_t v_t^T, o_t = S_t^T q_t.  Each head's o is divided by its root
+    mean square (``eps``, no weight), the heads side by side are multiplied by silu(W_g x),
+    then W_o.  Per request: S (float32)."""
+
+    kind: ClassVar[str] = "retention"
+    num_heads: int
+    head_dim: int
+    value_dim: int
+    decay: tuple
+    eps: float
+    position: object = None
+    names: Names = ()
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Several mixers side by side on the same input: ``branches`` = ((sub-name, mixer spec),
+    ...).  Each output is brought to unit root mean square over the model width (``eps``) and
+    multiplied by its own weight (tensor "<sub-name>.out" of the mixer, as it is stored); the
+    result is ``scale`` times their sum."""
+
+    kind: ClassVar[str] = "parallel_mixers"
+    branches: tuple
+    eps: float
+    scale: float = 0.5
+    out_name: str = "out"
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """A routed mixture of gated experts ("e0", "e1", ...), each down(act(gate x) * up x) of
+    ``expert_size`` features.  Router logits W_router x in float32; scores = softmax over all
+    experts; the ``top`` experts with the largest score + correction (a tensor of one number
+    per expert, with ``correction``) are chosen; their weights are their scores over the
+    chosen ones' sum (+ 1e-20).  ``shared_size``: a gated expert of that many features that
+    every token passes and whose output is added (None: none)."""
+
+    kind: ClassVar[str] = "moe"
+    experts: int
+    top: int
+    expert_size: int
+    shared_size: int | None = None
+    correction: bool = True
+    activation: str = "silu"
     names: Names = ()
 
 
@@ -202,6 +290,28 @@ class BlockSpec:
 
 
 @dataclass(frozen=True)
+class SandwichBlockSpec:
+    """A norm before and after each sublayer: x += mixer_post(mixer(mixer_norm(x)));
+    x += ffn_post(ffn(ffn_norm(x))).  ``ffn`` may be None: the layer then has no feed-forward
+    and neither of its norms."""
+
+    kind: ClassVar[str] = "sandwich_residual"
+    name: str
+    mixer: object
+    ffn: object
+    mixer_norm: object
+    mixer_post: object
+    ffn_norm: object = None
+    ffn_post: object = None
+    mixer_name: str = "mix"
+    ffn_name: str = "mlp"
+    mixer_norm_name: str = "norm1"
+    mixer_post_name: str = "norm1b"
+    ffn_norm_name: str = "norm2"
+    ffn_post_name: str = "norm2b"
+
+
+@dataclass(frozen=True)
 class ParallelBlockSpec:
     """h = norm(x); x += mixer(h) + ffn(h); then x = side(x, tokens) where there is one.
     One norm feeds both sublayers; ``ffn`` and ``side`` may be None."""
@@ -220,12 +330,15 @@ class ParallelBlockSpec:
 
 @dataclass(frozen=True)
 class TokenEmbeddingSpec:
-    """x = table[token id] * scale."""
+    """x = table[token id] * scale; with ``norm`` (a norm spec, its tensors under
+    ``norm_name``), x = norm(x) after that."""
 
     kind: ClassVar[str] = "token_lookup"
     vocab_size: int
     scale: float = 1.0
     names: Names = ()
+    norm: object = None
+    norm_name: str = "embed.norm"
 
 
 @dataclass(frozen=True)
@@ -245,11 +358,14 @@ class PairHashEmbeddingSpec:
 
 @dataclass(frozen=True)
 class LinearHeadSpec:
-    """logits = x @ W.T, no bias."""
+    """logits = (x @ W.T) * scale, no bias; with ``softcap``, logits <- softcap * tanh(logits /
+    softcap) after that."""
 
     kind: ClassVar[str] = "linear"
     vocab_size: int
     names: Names = ()
+    scale: float = 1.0
+    softcap: float | None = None
 
 
 @dataclass(frozen=True)
@@ -258,12 +374,17 @@ class ScheduleEntry:
     cache this run reads instead of owning one; None means it owns its cache.
     Before the run, ``add_embedding`` adds the embedding's output (the stream as it
     was before the first block) to the stream, and ``add_vector`` = (tensor, row)
-    adds row `row` of a tensor that the model declares in ``stream_vectors``."""
+    adds row `row` of a tensor that the model declares in ``stream_vectors``.
+    ``depth_average`` names a tensor of (position + 2) numbers c: with X_0 the embedding's
+    output and X_(k+1) what run k leaves, the stream that goes on after this run (position i)
+    is sum_j c[j] X_j, j = 0 .. i + 1; X_(i+1) itself is the run's result before that sum.
+    Either every entry of a schedule has one or none has."""
 
     block: int
     cache_of: int | None = None
     add_embedding: bool = False
     add_vector: tuple | None = None
+    depth_average: str | None = None
 
 
 @dataclass(frozen=True)
@@ -303,6 +424,9 @@ class ModelSpec:
             object.__setattr__(
                 self, "schedule", tuple(ScheduleEntry(i) for i in range(len(self.blocks)))
             )
+        averaged = [e.depth_average is not None for e in self.schedule]
+        if any(averaged) and not all(averaged):
+            raise ValueError("a depth average needs every run's result: every schedule entry must name one")
         for pos, entry in enumerate(self.schedule):
             if not 0 <= entry.block < len(self.blocks):
                 raise ValueError(f"schedule[{pos}] names block {entry.block}, which does not exist")

@@ -273,10 +273,90 @@ int shk_mlstm_scan(const float* proj, int ld, int q_off, int k_off, int v_off, i
                    const float* i_bias, const float* f_bias, float cap, float q_scale, int num_seqs,
                    int heads, int dim, int v_dim, const int32_t* positions, const int32_t* cu_q,
                    const int32_t* slots, float* state, long long slot_stride, float* out, void* stream);
-// out[t, h, :] = o[t, h, :] * rsqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gate[t, h, :]);
-// o float32 [n, heads * v_dim], gate float32 rows gate_ld apart, out of `dtype`.
+// out[t, h, :] = o[t, h, :] * rsqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * g(gate[t, h, :]);
+// o float32 [n, heads * v_dim], gate float32 rows gate_ld apart, out of `dtype`.  weight may be
+// null (none); gate_act 0: g is the sigmoid, 1: SiLU.
 int shk_headnorm_gate(const float* o, const float* gate, int gate_ld, const float* weight, float eps,
-                      void* out, int dtype, int n, int heads, int v_dim, void* stream);
+                      void* out, int dtype, int n, int heads, int v_dim, int gate_act, void* stream);
+
+// Layer norm with weight and bias around the float32 stream (layernorm.hip).  For each of n
+// rows r (row index rows[r] when `rows` is given, else r): x = resid[row]; with delta, x += d,
+// where d = delta[row] (of `dtype`, or float32 partial sums [delta_splits][resid_rows][hidden]),
+// and with dweight d is normed by itself first: d <- (d - mean(d)) / sqrt(var(d) + deps) * dweight
+// + dbias; with write_resid the sum is stored back.  With out, out[r] = (x - mean) / sqrt(var +
+// eps) * weight + bias, of `dtype`, or float32 with out_f32 (out may then be resid itself).  The
+// variance is the mean of the squared deviations; dbias and bias may be null.
+int shk_add_layernorm(float* resid, const void* delta, int delta_splits, const float* dweight,
+                      const float* dbias, float deps, const float* weight, const float* bias, float eps,
+                      void* out, int dtype, int out_f32, const int32_t* rows, int n, int hidden,
+                      int write_resid, int resid_rows, void* stream);
+// out[r, :] = sum over j < count of coef[j] * history[j * stride + r * hidden + :], added in
+// ascending j (float32).  With delta (as in shk_add_layernorm, always normed: dweight, dbias,
+// deps), the newest stream, j = count - 1, first gains the normed addend and is stored back.
+int shk_mix_history(float* history, long long stride, const float* coef, int count, float* out, int n,
+                    int hidden, const void* delta, int delta_splits, const float* dweight,
+                    const float* dbias, float deps, int dtype, void* stream);
+// x <- x * scale, then with cap > 0: x <- cap * tanh(x / cap); float32, elementwise.
+int shk_scale_softcap(float* x, long long numel, float scale, float cap, void* stream);
+
+// Attention with weights mixed across heads after the softmax (attention_talking.hip), over the
+// cache layouts of shk_attention: s_g = q_g . k * scale - r1[g] * ln(1 + r2[g] * distance) (r1,
+// r2 null: no bias); p_g = exp(s_g) / (exp(sink) [with has_sink] + sum exp(s_g)); head h applies
+// sum_g talk[h, g] p_g (talk null: the identity) to the values of its own key/value head.
+// scratch: shk_attention_talking_scratch_floats(n, heads, v_dim, nshare) floats; nshare > 1
+// shares every token's keys among that many workgroups.
+long long shk_attention_talking_scratch_floats(int n, int heads, int v_dim, int nshare);
+int shk_attention_talking(const void* q, int q_stride, void* out, int dtype, int n, int heads, int kv_heads,
+                          int head_dim, int v_dim, const int32_t* positions, const int32_t* token_seq,
+                          const int32_t* tables, int table_stride, const void* k_pool, const void* v_pool,
+                          int page_size, int num_pages, int window, int chunk, float scale,
+                          const float* r1, const float* r2, const float* talk, int has_sink, float sink,
+                          float* scratch, int nshare, void* stream);
+
+// The selective scan of Mamba and its causal convolution (ssm.hip).  A request's slot holds S
+// [inner, states] float32 and then the convolution's last taps - 1 inputs [(taps - 1), inner].
+// shk_conv_silu: y[t, c] = silu(bias[c] + sum_k taps[c, num_taps - 1 - k] * x[t - k, c]) over the
+// sequence's earlier inputs (rows of this step, else the slot's kept ones, zero before position 0).
+// shk_dt_softplus: dt[t, c] = softplus(b[c] + sum_r w[c, r] * low[t, r]), float32.
+// shk_selective_scan: S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n, y_c = sum_n S[c, n] C_n +
+// dskip_c x_c, out = y * silu(z); A = -exp(a_log); B and C are columns b_off, c_off of bc (float32);
+// `raw` are the convolution's inputs of the step, of which the slot keeps the last taps - 1.
+long long shk_selective_scan_state_floats(int inner, int states, int taps);
+int shk_conv_silu(const void* x, int ldx, const float* taps, const float* bias, int num_taps, int inner,
+                  const int32_t* positions, const int32_t* token_seq, const int32_t* cu_q,
+                  const int32_t* slots, const float* state, long long slot_stride, int states, void* y,
+                  int dtype, int n, void* stream);
+int shk_dt_softplus(const float* low, int ld, const float* w, const float* b, int rank, int inner,
+                    float* dt, int n, void* stream);
+int shk_selective_scan(const float* dt, const void* x, const float* bc, int ld_bc, int b_off, int c_off,
+                       const void* z, int ldz, const float* a_log, const float* dskip, int inner,
+                       int states, int num_taps, const void* raw, int ld_raw, const int32_t* positions,
+                       const int32_t* cu_q, const int32_t* slots, float* state, long long slot_stride,
+                       void* out, int dtype, int num_seqs, void* stream);
+
+// Retention (ssm.hip): per head S_t = decay[h] S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, over float32
+// projections at columns q_off, k_off ([heads, dim]) and v_off ([heads, v_dim]) of proj; a slot
+// holds S as [heads, v_dim, dim].  shk_rotate_half_rows turns the pairs (i, i + rot_dim / 2) of
+// every head of float32 rows in place by positions[t] * inv_freq[i] and multiplies the head by mult.
+long long shk_retention_state_floats(int heads, int dim, int v_dim);
+int shk_rotate_half_rows(float* x, int ld, int off, int heads, int dim, int rot_dim, const float* inv_freq,
+                         const int32_t* positions, float mult, int n, void* stream);
+int shk_retention_scan(const float* proj, int ld, int q_off, int k_off, int v_off, const float* decay,
+                       int num_seqs, int heads, int dim, int v_dim, const int32_t* positions,
+                       const int32_t* cu_q, const int32_t* slots, float* state, long long slot_stride,
+                       float* out, void* stream);
+
+// A routed mixture of gated experts (moe.hip).  shk_moe_route: softmax over the experts' logits
+// (float32 [n, ld]); the `top` largest of score + correction (null: none) are chosen [n, top],
+// their weights [n, top] are their scores over the chosen ones' sum (+ 1e-20).
+// shk_moe_experts: out[t] = add[t] (null: nothing) + sum_k weights[t, k] * W_down_e (act(W_gate_e
+// x_t) * (W_up_e x_t)), e = chosen[t, k]; matrices stacked row-major [experts, ff, width] and
+// [experts, width, ff]; act_buf [n * top, ff]; all of `dtype`; act 1 SiLU, 2 GELU (tanh form).
+int shk_moe_route(const float* logits, int ld, const float* correction, int experts, int top,
+                  int32_t* chosen, float* weights, int n, void* stream);
+int shk_moe_experts(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
+                    const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
+                    int dtype, int n, int width, int ff, int experts, int top, int act, void* stream);
 
 // out = a_pos z^2 + z / 2 where z > 0, a_neg (exp(z) - 1 - z) + z / 2 elsewhere; elementwise.
 int shk_xielu(const void* x, void* out, int dtype, long long numel, float a_pos, float a_neg, void* stream);

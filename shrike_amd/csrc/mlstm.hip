@@ -173,7 +173,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
     headnorm_gate_kernel(const float* __restrict__ o, const float* __restrict__ gate, int gate_ld,
                          const float* __restrict__ weight, float eps, T* __restrict__ out, int n, int heads,
-                         int v_dim) {
+                         int v_dim, int gate_act) {
   const int unit = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   if (unit >= n * heads) return;
@@ -185,8 +185,8 @@ __global__ void __launch_bounds__(256)
   const float* g = gate + static_cast<size_t>(t) * gate_ld + h * v_dim;
   T* y = out + (static_cast<size_t>(t) * heads + h) * v_dim;
   for (int d = lane; d < v_dim; d += kWave) {
-    const float s = 1.f / (1.f + expf(-g[d]));
-    y[d] = from_float<T>(x[d] * r * weight[h * v_dim + d] * s);
+    const float s = (gate_act == 1 ? g[d] : 1.f) / (1.f + expf(-g[d]));
+    y[d] = from_float<T>(x[d] * r * (weight ? weight[h * v_dim + d] : 1.f) * s);
   }
 }
 
@@ -235,19 +235,20 @@ extern "C" int shk_mlstm_scan(const float* proj, int ld, int q_off, int k_off, i
 }
 
 extern "C" int shk_headnorm_gate(const float* o, const float* gate, int gate_ld, const float* weight, float eps,
-                                 void* out, int dtype, int n, int heads, int v_dim, void* stream) {
+                                 void* out, int dtype, int n, int heads, int v_dim, int gate_act, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "headnorm_gate: unknown dtype %d", dtype);
+  SHK_REQUIRE(gate_act == 0 || gate_act == 1, "headnorm_gate: unknown gate %d (0: sigmoid, 1: SiLU)", gate_act);
   SHK_REQUIRE(n >= 0 && heads > 0 && v_dim > 0 && gate_ld >= heads * v_dim, "headnorm_gate: bad sizes n=%d heads=%d v_dim=%d gate_ld=%d",
               n, heads, v_dim, gate_ld);
   if (n == 0) return 0;
-  SHK_REQUIRE(o && gate && weight && out, "headnorm_gate: null pointer");
+  SHK_REQUIRE(o && gate && out, "headnorm_gate: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long long units = static_cast<long long>(n) * heads;
   const int grid = static_cast<int>((units + 3) / 4);
   if (dtype == kF32)
-    headnorm_gate_kernel<float><<<grid, 256, 0, s>>>(o, gate, gate_ld, weight, eps, static_cast<float*>(out), n, heads, v_dim);
+    headnorm_gate_kernel<float><<<grid, 256, 0, s>>>(o, gate, gate_ld, weight, eps, static_cast<float*>(out), n, heads, v_dim, gate_act);
   else
-    headnorm_gate_kernel<bf16><<<grid, 256, 0, s>>>(o, gate, gate_ld, weight, eps, static_cast<bf16*>(out), n, heads, v_dim);
+    headnorm_gate_kernel<bf16><<<grid, 256, 0, s>>>(o, gate, gate_ld, weight, eps, static_cast<bf16*>(out), n, heads, v_dim, gate_act);
   SHK_LAUNCH_CHECK("headnorm_gate");
   return 0;
 }

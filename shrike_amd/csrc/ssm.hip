@@ -1,0 +1,385 @@
+// Recurrent mixers whose state is a fixed-size tensor per request: the selective
+// scan of Mamba (with its short causal convolution) and retention (linear
+// attention with a fixed decay per head).  A sequence's tokens of the step are
+// walked in order, whether they are a prompt's portion or one decoded token, so
+// a position's result does not depend on how the prompt was cut.  All state and
+// everything in the recurrences is float32.  A state is taken as zero where the
+// sequence's first row of the step is at position 0: a slot that another request
+// left full starts from nothing.
+//
+// Selective scan, per channel c and state n:
+//   S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n;   y_c = sum_n S[c, n] C_n + D_c x_c
+// with dt = softplus(W_dt low + b) per channel and A = -exp(A_log).
+// A request's slot holds S [inner, state] and then the convolution's last taps - 1
+// inputs [(taps - 1), inner], oldest first.
+//
+// Retention, per head:  S_t = decay S_(t-1) + k_t v_t^T;  o_t = S_t^T q_t.
+// A request's slot holds S as [heads, v_dim, dim].
+#include "api.h"
+#include "common.h"
+
+namespace shk {
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// y[t, c] = silu(bias[c] + sum_k taps[c, K - 1 - k] * x(t - k, c)): x(t - k) is a row of this
+// step where the sequence's portion reaches that far back, else the slot's kept input of
+// that position, else (before the sequence's start) zero.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    conv_silu_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ taps, const float* __restrict__ bias,
+                     int K, int inner, const int32_t* __restrict__ positions, const int32_t* __restrict__ token_seq,
+                     const int32_t* __restrict__ cu_q, const int32_t* __restrict__ slots,
+                     const float* __restrict__ state, long long slot_stride, long long tail_off,
+                     T* __restrict__ y) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= inner) return;
+  const int seq = token_seq[t];
+  const int pos = positions[t];
+  const int first = cu_q[seq];  // the sequence's first row of the step
+  const float* tail = state + static_cast<size_t>(slots[seq]) * slot_stride + tail_off;
+  float acc = bias[c];
+  for (int k = K - 1; k >= 0; --k) {  // oldest input first
+    float v = 0.f;
+    if (pos - k >= 0) {
+      if (t - k >= first) {
+        v = to_float(x[static_cast<size_t>(t - k) * ldx + c]);
+      } else {
+        // the slot keeps the inputs of the K - 1 positions before the step, oldest first:
+        // entry e holds position (start - (K - 1) + e), start = the position of row `first`
+        const int start = pos - (t - first);
+        const int e = (pos - k) - (start - (K - 1));
+        v = tail[static_cast<size_t>(e) * inner + c];
+      }
+    }
+    acc = fmaf(taps[c * K + (K - 1 - k)], v, acc);
+  }
+  y[static_cast<size_t>(t) * inner + c] = from_float<T>(silu_f(acc));
+}
+
+// dt[t, c] = softplus(b[c] + sum_r W[c, r] * low[t, r]) in float32
+__global__ void __launch_bounds__(256)
+    dt_softplus_kernel(const float* __restrict__ low, int ld, const float* __restrict__ w, const float* __restrict__ b,
+                       int rank, int inner, float* __restrict__ dt) {
+  extern __shared__ float lows[];
+  const int t = blockIdx.y;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) lows[r] = low[static_cast<size_t>(t) * ld + r];
+  __syncthreads();
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= inner) return;
+  float acc = b[c];
+  const float* wr = w + static_cast<size_t>(c) * rank;
+  for (int r = 0; r < rank; ++r) acc = fmaf(wr[r], lows[r], acc);
+  dt[static_cast<size_t>(t) * inner + c] = softplus_f(acc);
+}
+
+constexpr int kStatesPerLane = 8;
+
+// One sequence's tokens for a block of channels.  LANES lanes share a channel's states
+// (LANES * 8 >= states); a wavefront holds 64 / LANES channels.
+template <typename T, int LANES>
+__global__ void __launch_bounds__(256)
+    selective_scan_kernel(const float* __restrict__ dt, const T* __restrict__ x, const float* __restrict__ bc,
+                          int ld_bc, int b_off, int c_off, const T* __restrict__ z, int ldz,
+                          const float* __restrict__ a_log, const float* __restrict__ dskip, int inner, int states,
+                          int K, const T* __restrict__ raw, int ld_raw, const int32_t* __restrict__ positions,
+                          const int32_t* __restrict__ cu_q, const int32_t* __restrict__ slots,
+                          float* __restrict__ state, long long slot_stride, T* __restrict__ out) {
+  const int seq = blockIdx.y;
+  const int unit = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;  // channel
+  const int part = threadIdx.x % LANES;
+  if (unit >= inner) return;
+  const int c = unit;
+  const int first = cu_q[seq], last = cu_q[seq + 1];
+  if (last <= first) return;
+  float* slot = state + static_cast<size_t>(slots[seq]) * slot_stride;
+  float* srow = slot + static_cast<size_t>(c) * states;
+  const bool fresh = positions[first] == 0;
+  float S[kStatesPerLane], A[kStatesPerLane];
+#pragma unroll
+  for (int i = 0; i < kStatesPerLane; ++i) {
+    const int n = part * kStatesPerLane + i;
+    S[i] = (n < states && !fresh) ? srow[n] : 0.f;
+    A[i] = n < states ? -expf(a_log[static_cast<size_t>(c) * states + n]) : 0.f;
+  }
+  const float dc = dskip[c];
+  for (int t = first; t < last; ++t) {
+    const float step = dt[static_cast<size_t>(t) * inner + c];
+    const float xv = to_float(x[static_cast<size_t>(t) * inner + c]);
+    const float* bt = bc + static_cast<size_t>(t) * ld_bc + b_off;
+    const float* ct = bc + static_cast<size_t>(t) * ld_bc + c_off;
+    const float dx = step * xv;
+    float y = 0.f;
+#pragma unroll
+    for (int i = 0; i < kStatesPerLane; ++i) {
+      const int n = part * kStatesPerLane + i;
+      if (n < states) {
+        S[i] = fmaf(expf(step * A[i]), S[i], dx * bt[n]);
+        y = fmaf(S[i], ct[n], y);
+      }
+    }
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) y += __shfl_xor(y, off, kWave);
+    if (part == 0) {
+      y = fmaf(dc, xv, y);
+      const float g = to_float(z[static_cast<size_t>(t) * ldz + c]);
+      out[static_cast<size_t>(t) * inner + c] = from_float<T>(y * silu_f(g));
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kStatesPerLane; ++i) {
+    const int n = part * kStatesPerLane + i;
+    if (n < states) srow[n] = S[i];
+  }
+  // the convolution's kept inputs: the K - 1 positions before the next step, oldest first
+  if (part == 0 && K > 1) {
+    float* tail = slot + static_cast<size_t>(inner) * states;
+    const int count = last - first;
+    for (int e = 0; e < K - 1; ++e) {
+      const int back = (K - 1) - e;  // the input `back` positions before the next step
+      float v = 0.f;
+      if (back <= count) {
+        v = to_float(raw[static_cast<size_t>(last - back) * ld_raw + c]);
+      } else if (!fresh) {
+        v = tail[static_cast<size_t>(e + count) * inner + c];  // shifts up; e + count <= K - 2
+      }
+      tail[static_cast<size_t>(e) * inner + c] = v;
+    }
+  }
+}
+
+// Rotation of element pairs (i, i + rot_dim / 2) of every head of float32 rows, in place:
+// x[t, off + h * dim + e]; angle position * inv_freq[i]; all of the head is multiplied
+// by `mult` afterwards.
+__global__ void __launch_bounds__(256)
+    rotate_half_rows_kernel(float* __restrict__ x, int ld, int off, int heads, int dim, int rot_dim,
+                            const float* __restrict__ inv_freq, const int32_t* __restrict__ positions, float mult,
+                            int n) {
+  const int half = rot_dim / 2;
+  const int per_head = dim - half;  // a thread takes a pair, or one unrotated element
+  const long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (item >= static_cast<long long>(n) * heads * per_head) return;
+  const int e = static_cast<int>(item % per_head);
+  const int h = static_cast<int>((item / per_head) % heads);
+  const int t = static_cast<int>(item / (static_cast<long long>(per_head) * heads));
+  float* row = x + static_cast<size_t>(t) * ld + off + h * dim;
+  if (e < half) {
+    const float angle = static_cast<float>(positions[t]) * inv_freq[e];
+    const double wide = static_cast<double>(angle);
+    const double turns = rint(wide * 0.15915494309189535);
+    const float reduced = static_cast<float>(wide - turns * 6.283185307179586);
+    float sv, cv;
+    sincosf(reduced, &sv, &cv);
+    const float u = row[e], v = row[e + half];
+    row[e] = (u * cv - v * sv) * mult;
+    row[e + half] = (v * cv + u * sv) * mult;
+  } else {
+    row[e + half] *= mult;  // elements from rot_dim on
+  }
+}
+
+constexpr int kRowsPerLane = 16;
+
+// One sequence's tokens for one (head, value column); LANES lanes share the column's rows
+// of S (LANES * 16 >= dim).
+template <int LANES>
+__global__ void __launch_bounds__(256)
+    retention_scan_kernel(const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
+                          const float* __restrict__ decay, int heads, int dim, int v_dim,
+                          const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
+                          const int32_t* __restrict__ slots, float* __restrict__ state, long long slot_stride,
+                          float* __restrict__ out) {
+  const int seq = blockIdx.y;
+  const int unit = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;  // (head, column)
+  const int part = threadIdx.x % LANES;
+  if (unit >= heads * v_dim) return;
+  const int h = unit / v_dim, col = unit % v_dim;
+  const int first = cu_q[seq], last = cu_q[seq + 1];
+  if (last <= first) return;
+  float* srow = state + static_cast<size_t>(slots[seq]) * slot_stride + static_cast<size_t>(unit) * dim;
+  const bool fresh = positions[first] == 0;
+  float S[kRowsPerLane];
+#pragma unroll
+  for (int i = 0; i < kRowsPerLane; ++i) {
+    const int d = part * kRowsPerLane + i;
+    S[i] = (d < dim && !fresh) ? srow[d] : 0.f;
+  }
+  const float a = decay[h];
+  for (int t = first; t < last; ++t) {
+    const float* row = proj + static_cast<size_t>(t) * ld;
+    const float* qt = row + q_off + h * dim;
+    const float* kt = row + k_off + h * dim;
+    const float vv = row[v_off + h * v_dim + col];
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRowsPerLane; ++i) {
+      const int d = part * kRowsPerLane + i;
+      if (d < dim) {
+        S[i] = fmaf(a, S[i], kt[d] * vv);
+        o = fmaf(S[i], qt[d], o);
+      }
+    }
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) o += __shfl_xor(o, off, kWave);
+    if (part == 0) out[static_cast<size_t>(t) * heads * v_dim + unit] = o;
+  }
+#pragma unroll
+  for (int i = 0; i < kRowsPerLane; ++i) {
+    const int d = part * kRowsPerLane + i;
+    if (d < dim) srow[d] = S[i];
+  }
+}
+
+inline int lanes_for(int items, int per_lane) {
+  int lanes = 1;
+  while (lanes * per_lane < items) lanes *= 2;
+  return lanes;
+}
+
+}  // namespace shk
+
+using namespace shk;
+
+extern "C" long long shk_selective_scan_state_floats(int inner, int states, int taps) {
+  return static_cast<long long>(inner) * states + static_cast<long long>(taps > 1 ? taps - 1 : 0) * inner;
+}
+
+extern "C" int shk_conv_silu(const void* x, int ldx, const float* taps, const float* bias, int num_taps, int inner,
+                             const int32_t* positions, const int32_t* token_seq, const int32_t* cu_q,
+                             const int32_t* slots, const float* state, long long slot_stride, int states, void* y,
+                             int dtype, int n, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "conv_silu: unknown dtype %d", dtype);
+  SHK_REQUIRE(n >= 0 && inner > 0 && num_taps >= 1 && num_taps <= 64 && ldx >= inner && states > 0,
+              "conv_silu: bad sizes n=%d inner=%d taps=%d", n, inner, num_taps);
+  SHK_REQUIRE(slot_stride >= shk_selective_scan_state_floats(inner, states, num_taps),
+              "conv_silu: a slot of %lld floats does not hold the state", slot_stride);
+  if (n == 0) return 0;
+  SHK_REQUIRE(n <= 65535, "conv_silu: at most 65535 tokens a call, got %d", n);
+  SHK_REQUIRE(x && taps && bias && positions && token_seq && cu_q && slots && state && y, "conv_silu: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid((inner + 255) / 256, n);
+  const long long tail_off = static_cast<long long>(inner) * states;
+  if (dtype == kF32)
+    conv_silu_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(x), ldx, taps, bias, num_taps, inner,
+                                                 positions, token_seq, cu_q, slots, state, slot_stride, tail_off,
+                                                 static_cast<float*>(y));
+  else
+    conv_silu_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(x), ldx, taps, bias, num_taps, inner,
+                                                positions, token_seq, cu_q, slots, state, slot_stride, tail_off,
+                                                static_cast<bf16*>(y));
+  SHK_LAUNCH_CHECK("conv_silu");
+  return 0;
+}
+
+extern "C" int shk_dt_softplus(const float* low, int ld, const float* w, const float* b, int rank, int inner,
+                               float* dt, int n, void* stream) {
+  SHK_REQUIRE(n >= 0 && inner > 0 && rank > 0 && rank <= 8192 && ld >= rank, "dt_softplus: bad sizes n=%d inner=%d rank=%d",
+              n, inner, rank);
+  if (n == 0) return 0;
+  SHK_REQUIRE(n <= 65535, "dt_softplus: at most 65535 tokens a call, got %d", n);
+  SHK_REQUIRE(low && w && b && dt, "dt_softplus: null pointer");
+  dim3 grid((inner + 255) / 256, n);
+  dt_softplus_kernel<<<grid, 256, rank * sizeof(float), static_cast<hipStream_t>(stream)>>>(low, ld, w, b, rank, inner,
+                                                                                           dt);
+  SHK_LAUNCH_CHECK("dt_softplus");
+  return 0;
+}
+
+extern "C" int shk_selective_scan(const float* dt, const void* x, const float* bc, int ld_bc, int b_off, int c_off,
+                                  const void* z, int ldz, const float* a_log, const float* dskip, int inner,
+                                  int states, int num_taps, const void* raw, int ld_raw, const int32_t* positions,
+                                  const int32_t* cu_q, const int32_t* slots, float* state, long long slot_stride,
+                                  void* out, int dtype, int num_seqs, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "selective_scan: unknown dtype %d", dtype);
+  SHK_REQUIRE(num_seqs >= 0 && inner > 0 && states > 0 && states <= 64 * kStatesPerLane && num_taps >= 1,
+              "selective_scan: bad sizes seqs=%d inner=%d states=%d", num_seqs, inner, states);
+  SHK_REQUIRE(b_off >= 0 && c_off >= 0 && b_off + states <= ld_bc && c_off + states <= ld_bc && ldz >= inner &&
+                  ld_raw >= inner,
+              "selective_scan: columns do not fit their rows");
+  SHK_REQUIRE(slot_stride >= shk_selective_scan_state_floats(inner, states, num_taps),
+              "selective_scan: a slot of %lld floats does not hold the state", slot_stride);
+  if (num_seqs == 0) return 0;
+  SHK_REQUIRE(num_seqs <= 65535, "selective_scan: at most 65535 sequences a call");
+  SHK_REQUIRE(dt && x && bc && z && a_log && dskip && raw && positions && cu_q && slots && state && out,
+              "selective_scan: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int lanes = lanes_for(states, kStatesPerLane);
+#define SHK_GO(T, L)                                                                                                 \
+  selective_scan_kernel<T, L><<<dim3((inner + 256 / L - 1) / (256 / L), num_seqs), 256, 0, s>>>(                     \
+      dt, static_cast<const T*>(x), bc, ld_bc, b_off, c_off, static_cast<const T*>(z), ldz, a_log, dskip, inner,     \
+      states, num_taps, static_cast<const T*>(raw), ld_raw, positions, cu_q, slots, state, slot_stride,              \
+      static_cast<T*>(out))
+#define SHK_LANES(T)                                                                                                 \
+  switch (lanes) {                                                                                                   \
+    case 1: SHK_GO(T, 1); break;                                                                                     \
+    case 2: SHK_GO(T, 2); break;                                                                                     \
+    case 4: SHK_GO(T, 4); break;                                                                                     \
+    case 8: SHK_GO(T, 8); break;                                                                                     \
+    case 16: SHK_GO(T, 16); break;                                                                                   \
+    case 32: SHK_GO(T, 32); break;                                                                                   \
+    default: SHK_GO(T, 64); break;                                                                                   \
+  }
+  if (dtype == kF32) {
+    SHK_LANES(float)
+  } else {
+    SHK_LANES(bf16)
+  }
+#undef SHK_LANES
+#undef SHK_GO
+  SHK_LAUNCH_CHECK("selective_scan");
+  return 0;
+}
+
+extern "C" int shk_rotate_half_rows(float* x, int ld, int off, int heads, int dim, int rot_dim, const float* inv_freq,
+                                    const int32_t* positions, float mult, int n, void* stream) {
+  SHK_REQUIRE(n >= 0 && heads > 0 && dim > 0 && rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= dim && off >= 0 &&
+                  off + heads * dim <= ld,
+              "rotate_half_rows: bad sizes heads=%d dim=%d rot_dim=%d", heads, dim, rot_dim);
+  if (n == 0) return 0;
+  SHK_REQUIRE(x && positions && (rot_dim == 0 || inv_freq), "rotate_half_rows: null pointer");
+  const long long items = static_cast<long long>(n) * heads * (dim - rot_dim / 2);
+  rotate_half_rows_kernel<<<static_cast<unsigned>((items + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      x, ld, off, heads, dim, rot_dim, inv_freq, positions, mult, n);
+  SHK_LAUNCH_CHECK("rotate_half_rows");
+  return 0;
+}
+
+extern "C" long long shk_retention_state_floats(int heads, int dim, int v_dim) {
+  return static_cast<long long>(heads) * v_dim * dim;
+}
+
+extern "C" int shk_retention_scan(const float* proj, int ld, int q_off, int k_off, int v_off, const float* decay,
+                                  int num_seqs, int heads, int dim, int v_dim, const int32_t* positions,
+                                  const int32_t* cu_q, const int32_t* slots, float* state, long long slot_stride,
+                                  float* out, void* stream) {
+  SHK_REQUIRE(num_seqs >= 0 && heads > 0 && dim > 0 && dim <= 64 * kRowsPerLane && v_dim > 0,
+              "retention_scan: bad sizes seqs=%d heads=%d dim=%d v_dim=%d", num_seqs, heads, dim, v_dim);
+  SHK_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= ld && k_off + heads * dim <= ld &&
+                  v_off + heads * v_dim <= ld,
+              "retention_scan: columns do not fit rows of %d", ld);
+  SHK_REQUIRE(slot_stride >= shk_retention_state_floats(heads, dim, v_dim),
+              "retention_scan: a slot of %lld floats does not hold the state", slot_stride);
+  if (num_seqs == 0) return 0;
+  SHK_REQUIRE(num_seqs <= 65535, "retention_scan: at most 65535 sequences a call");
+  SHK_REQUIRE(proj && decay && positions && cu_q && slots && state && out, "retention_scan: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int lanes = lanes_for(dim, kRowsPerLane);
+  const int units = heads * v_dim;
+#define SHK_GO(L)                                                                                              \
+  retention_scan_kernel<L><<<dim3((units + 256 / L - 1) / (256 / L), num_seqs), 256, 0, s>>>(                  \
+      proj, ld, q_off, k_off, v_off, decay, heads, dim, v_dim, positions, cu_q, slots, state, slot_stride, out)
+  switch (lanes) {
+    case 1: SHK_GO(1); break;
+    case 2: SHK_GO(2); break;
+    case 4: SHK_GO(4); break;
+    case 8: SHK_GO(8); break;
+    case 16: SHK_GO(16); break;
+    case 32: SHK_GO(32); break;
+    default: SHK_GO(64); break;
+  }
+#undef SHK_GO
+  SHK_LAUNCH_CHECK("retention_scan");
+  return 0;
+}

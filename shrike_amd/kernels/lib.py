@@ -53,7 +53,20 @@ _SIGNATURES = {
     "shk_latent_attention_bf16": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P, _I, _I, _P],
     "shk_gemm_batched": [_P, _P, _P, _I, _I, _I, _I, _I, _I, c_longlong, c_longlong, c_longlong, _I, _P],
     "shk_mlstm_scan": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _F, _I, _I, _I, _I, _P, _P, _P, _P, c_longlong, _P, _P],
-    "shk_headnorm_gate": [_P, _P, _I, _P, _F, _P, _I, _I, _I, _I, _P],
+    "shk_headnorm_gate": [_P, _P, _I, _P, _F, _P, _I, _I, _I, _I, _I, _P],
+    "shk_add_layernorm": [_P, _P, _I, _P, _P, _F, _P, _P, _F, _P, _I, _I, _P, _I, _I, _I, _I, _P],
+    "shk_mix_history": [_P, c_longlong, _P, _I, _P, _I, _I, _P, _I, _P, _P, _F, _I, _P],
+    "shk_scale_softcap": [_P, c_longlong, _F, _F, _P],
+    "shk_attention_talking": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _P, _P,
+                              _P, _I, _F, _P, _I, _P],
+    "shk_conv_silu": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, c_longlong, _I, _P, _I, _I, _P],
+    "shk_dt_softplus": [_P, _I, _P, _P, _I, _I, _P, _I, _P],
+    "shk_selective_scan": [_P, _P, _P, _I, _I, _I, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, c_longlong,
+                           _P, _I, _I, _P],
+    "shk_rotate_half_rows": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _I, _P],
+    "shk_retention_scan": [_P, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, c_longlong, _P, _P],
+    "shk_moe_route": [_P, _I, _P, _I, _I, _P, _P, _I, _P],
+    "shk_moe_experts": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "shk_xielu": [_P, _P, _I, c_longlong, _F, _F, _P],
     "shk_embed_pairs": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],
@@ -120,6 +133,12 @@ def load():
         raw.shk_mlstm_state_floats.argtypes = [_I, _I, _I]
         raw.shk_mlstm_state_floats.restype = c_longlong
         lib.shk_mlstm_state_floats = raw.shk_mlstm_state_floats
+        for name, argtypes in (("shk_attention_talking_scratch_floats", [_I, _I, _I, _I]),
+                               ("shk_selective_scan_state_floats", [_I, _I, _I]),
+                               ("shk_retention_state_floats", [_I, _I, _I])):
+            fn = getattr(raw, name)
+            fn.argtypes, fn.restype = argtypes, c_longlong
+            setattr(lib, name, fn)
         raw.shk_sample_scratch_floats.argtypes = [_I, _I]
         raw.shk_sample_scratch_floats.restype = c_longlong
         lib.shk_sample_scratch_floats = raw.shk_sample_scratch_floats

@@ -653,18 +653,266 @@ def mlstm_scan(proj, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_s
         _dev(slots, "slots", torch.int32), _dev(state, "state"), state.stride(0), _dev(out, "out"), _stream()))
 
 
-def headnorm_gate(o, gate, weight, eps, out, heads, v_dim) -> None:
-    """out[t, h] = o[t, h] / rms(o[t, h]) * weight[h] * sigmoid(gate[t, h]); o float32 [n, heads * v_dim],
-    gate float32 rows (a view with a row stride is fine), out of the compute dtype."""
+def headnorm_gate(o, gate, weight, eps, out, heads, v_dim, gate_act: str = "sigmoid") -> None:
+    """out[t, h] = o[t, h] / rms(o[t, h]) * weight[h] * g(gate[t, h]); o float32 [n, heads * v_dim],
+    gate float32 rows (a view with a row stride is fine), out of the compute dtype.  weight
+    None: none; gate_act "sigmoid" or "silu"."""
     _rows(gate, "headnorm_gate gate")
     n = o.shape[0]
     if o.dtype != torch.float32 or gate.dtype != torch.float32 or not o.is_contiguous() or not out.is_contiguous() \
             or tuple(o.shape) != (n, heads * v_dim) or tuple(out.shape) != (n, heads * v_dim) \
-            or gate.shape[0] != n or gate.shape[1] < heads * v_dim or weight.numel() != heads * v_dim:
+            or gate.shape[0] != n or gate.shape[1] < heads * v_dim \
+            or (weight is not None and weight.numel() != heads * v_dim):
         raise KernelError("headnorm_gate: o, gate float32 [n, heads * v_dim], out alike in the compute dtype")
+    if gate_act not in ("sigmoid", "silu"):
+        raise KernelError(f"headnorm_gate: unknown gate {gate_act!r}")
     check(load().shk_headnorm_gate(_dev(o, "o"), _dev(gate, "gate"), gate.stride(0),
-                                   _dev(weight, "weight", torch.float32), float(eps), _dev(out, "out"),
-                                   dtype_code(out.dtype), n, heads, v_dim, _stream()))
+                                   None if weight is None else _dev(weight, "weight", torch.float32), float(eps),
+                                   _dev(out, "out"), dtype_code(out.dtype), n, heads, v_dim,
+                                   int(gate_act == "silu"), _stream()))
+
+
+def _delta_any(delta, n, hidden, dtype, who: str):
+    """(address, splits) of an addend [n, hidden]: a tensor of the compute dtype or a SplitSum."""
+    if isinstance(delta, SplitSum):
+        if delta.bias is not None or tuple(delta.shape) != (n, hidden) or delta.parts.dtype != torch.float32 \
+                or not delta.parts.is_contiguous():
+            raise KernelError(f"{who}: partial sums must be contiguous float32 [splits, n, hidden] without bias")
+        return _dev(delta.parts, "delta"), delta.parts.shape[0]
+    if delta.dtype != dtype or not delta.is_contiguous() or tuple(delta.shape) != (n, hidden):
+        raise KernelError(f"{who}: an addend must be contiguous [n, hidden] of the compute dtype")
+    return _dev(delta, "delta"), 0
+
+
+def _f32vec(t, hidden, who):
+    if t is None:
+        return None
+    if t.dtype != torch.float32 or t.numel() != hidden or not t.is_contiguous():
+        raise KernelError(f"{who}: expected a contiguous float32 vector of {hidden}")
+    return _dev(t, who)
+
+
+def add_layernorm(resid, delta=None, dnorm=None, weight=None, bias=None, eps: float = 0.0, out=None, rows=None,
+                  write_resid: bool = True, dtype=None) -> None:
+    """Layer norm (weight, bias, variance as the mean squared deviation) around the float32
+    stream.  resid [N, hidden] gains `delta` (a product's output, tensor or SplitSum), which with
+    dnorm = (weight, bias, eps) is normed by itself first; `out` [n, hidden] (the compute dtype,
+    or float32; it may be resid itself) receives the layer norm of the sum.  rows: int32 row
+    indices, out[r] then belongs to resid[rows[r]]."""
+    hidden = resid.shape[1]
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("add_layernorm: resid must be contiguous float32")
+    n = resid.shape[0] if rows is None else rows.shape[0]
+    if out is not None:
+        dtype = out.dtype if out.dtype != torch.float32 or dtype is None else dtype
+        if tuple(out.shape) != (n, hidden) or not out.is_contiguous():
+            raise KernelError("add_layernorm: out must be contiguous [rows, hidden]")
+    if dtype is None:
+        dtype = delta.dtype if isinstance(delta, torch.Tensor) else torch.float32
+    d_ptr, d_splits = (None, 0) if delta is None else _delta_any(delta, resid.shape[0], hidden, dtype, "add_layernorm")
+    dw, db, deps = (None, None, 0.0) if dnorm is None else dnorm
+    check(load().shk_add_layernorm(
+        _dev(resid, "resid"), d_ptr, d_splits, _f32vec(dw, hidden, "dweight"), _f32vec(db, hidden, "dbias"),
+        float(deps), _f32vec(weight, hidden, "weight"), _f32vec(bias, hidden, "bias"), float(eps),
+        None if out is None else _dev(out, "out"), dtype_code(dtype),
+        int(out is not None and out.dtype == torch.float32),
+        None if rows is None else _dev(rows, "rows", torch.int32), n, hidden, int(bool(write_resid)),
+        resid.shape[0], _stream()))
+
+
+def mix_history(history, coef, count: int, out, delta=None, dnorm=None, dtype=None) -> None:
+    """out = sum_j coef[j] * history[j], j < count (float32 [slots, n, hidden] -> [n, hidden]); with
+    delta and dnorm = (weight, bias, eps), history[count - 1] first gains the normed addend."""
+    if history.dim() != 3 or history.dtype != torch.float32 or not history.is_contiguous() or count > history.shape[0]:
+        raise KernelError("mix_history: history must be contiguous float32 [slots >= count, n, hidden]")
+    _, n, hidden = history.shape
+    if tuple(out.shape) != (n, hidden) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise KernelError("mix_history: out must be contiguous float32 [n, hidden]")
+    if coef.dtype != torch.float32 or coef.numel() < count or not coef.is_contiguous():
+        raise KernelError("mix_history: coef must hold count float32 values")
+    if dtype is None:
+        dtype = delta.dtype if isinstance(delta, torch.Tensor) else torch.float32
+    d_ptr, d_splits = (None, 0) if delta is None else _delta_any(delta, n, hidden, dtype, "mix_history")
+    dw, db, deps = (None, None, 0.0) if dnorm is None else dnorm
+    check(load().shk_mix_history(_dev(history, "history"), history.stride(0), _dev(coef, "coef"), count,
+                                 _dev(out, "out"), n, hidden, d_ptr, d_splits, _f32vec(dw, hidden, "dweight"),
+                                 _f32vec(db, hidden, "dbias"), float(deps), dtype_code(dtype), _stream()))
+
+
+def scale_softcap(x, scale: float, cap) -> None:
+    """x <- cap * tanh(x * scale / cap) (cap None: x * scale), float32, in place."""
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("scale_softcap: expected a contiguous float32 tensor")
+    check(load().shk_scale_softcap(_dev(x, "x"), x.numel(), float(scale), float(cap or 0.0), _stream()))
+
+
+def attention_talking_scratch_floats(n: int, heads: int, v_dim: int, nshare: int) -> int:
+    return int(load().shk_attention_talking_scratch_floats(n, heads, v_dim, nshare))
+
+
+def attention_talking(q, out, heads, kv_heads, head_dim, v_dim, positions, token_seq, tables, k_pool, v_pool,
+                      page_size, window, scale, scratch, chunk=None, r1=None, r2=None, talk=None, sink=None,
+                      nshare: int = 1) -> None:
+    """Attention with a distance bias r1 ln(1 + r2 distance) taken off the scores, a sink of
+    score `sink` (None: none) in the denominator, and the softmax weights mixed across heads by
+    talk [heads, heads] before they meet the values.  q rows [n, >= heads * head_dim]; out
+    [n, heads * v_dim]; scratch float32 of attention_talking_scratch_floats(...)."""
+    _rows(q, "attention_talking q")
+    n = q.shape[0]
+    if tuple(out.shape) != (n, heads * v_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("attention_talking: out must be contiguous [n, heads * v_dim] of q's dtype")
+    for name, t, count in (("r1", r1, heads), ("r2", r2, heads), ("talk", talk, heads * heads)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != count or not t.is_contiguous()):
+            raise KernelError(f"attention_talking: {name} must be contiguous float32 of {count} values")
+    if scratch.dtype != torch.float32 or scratch.numel() < attention_talking_scratch_floats(n, heads, v_dim, nshare):
+        raise KernelError("attention_talking: scratch is too small")
+    _check_pools("attention_talking", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size, v_dim)
+    check(load().shk_attention_talking(
+        _dev(q, "q"), q.stride(0), _dev(out, "out"), dtype_code(q.dtype), n, heads, kv_heads, head_dim, v_dim,
+        _dev(positions, "positions", torch.int32), _dev(token_seq, "token_seq", torch.int32),
+        _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"),
+        page_size, k_pool.shape[0], int(window or 0), int(chunk or 0), float(scale),
+        None if r1 is None else _dev(r1, "r1"), None if r2 is None else _dev(r2, "r2"),
+        None if talk is None else _dev(talk, "talk"), int(sink is not None), float(sink or 0.0),
+        _dev(scratch, "scratch"), int(nshare), _stream()))
+
+
+def selective_scan_state_floats(inner: int, states: int, taps: int) -> int:
+    return int(load().shk_selective_scan_state_floats(inner, states, taps))
+
+
+def _state2d(state, who):
+    if state.dim() != 2 or state.dtype != torch.float32 or state.stride(1) != 1:
+        raise KernelError(f"{who}: state must be float32 [slots, floats]")
+
+
+def conv_silu(x, taps, bias, positions, token_seq, cu_q, slots, state, states: int, y) -> None:
+    """y = silu(causal convolution of x's channels over each sequence's inputs): x rows [n, >= inner]
+    (a view is fine), taps float32 [inner, K] whose last column meets the current token, the
+    slot's kept inputs for the positions before the step."""
+    _rows(x, "conv_silu x")
+    n, inner = y.shape
+    if y.dtype != x.dtype or not y.is_contiguous() or x.shape[0] != n or x.shape[1] < inner:
+        raise KernelError("conv_silu: y must be contiguous [n, inner] of x's dtype")
+    if taps.dtype != torch.float32 or taps.dim() != 2 or taps.shape[0] != inner or not taps.is_contiguous() \
+            or bias.dtype != torch.float32 or bias.numel() != inner:
+        raise KernelError("conv_silu: taps float32 [inner, K], bias float32 [inner]")
+    _state2d(state, "conv_silu")
+    check(load().shk_conv_silu(_dev(x, "x"), x.stride(0), _dev(taps, "taps"), _dev(bias, "bias"), taps.shape[1], inner,
+                               _dev(positions, "positions", torch.int32), _dev(token_seq, "token_seq", torch.int32),
+                               _dev(cu_q, "cu_q", torch.int32), _dev(slots, "slots", torch.int32), _dev(state, "state"),
+                               state.stride(0), states, _dev(y, "y"), dtype_code(y.dtype), n, _stream()))
+
+
+def dt_softplus(low, w, b, dt) -> None:
+    """dt = softplus(low[:, :rank] @ w.T + b) in float32; low rows may be a view."""
+    _rows(low, "dt_softplus low")
+    n, inner = dt.shape
+    rank = w.shape[1]
+    if low.dtype != torch.float32 or dt.dtype != torch.float32 or w.dtype != torch.float32 or b.dtype != torch.float32 \
+            or not dt.is_contiguous() or not w.is_contiguous() or tuple(w.shape) != (inner, rank) or b.numel() != inner \
+            or low.shape[0] != n or low.shape[1] < rank:
+        raise KernelError("dt_softplus: float32 low [n, >= rank], w [inner, rank], b [inner], dt [n, inner]")
+    check(load().shk_dt_softplus(_dev(low, "low"), low.stride(0), _dev(w, "w"), _dev(b, "b"), rank, inner,
+                                 _dev(dt, "dt"), n, _stream()))
+
+
+def selective_scan(dt, x, bc, b_off, c_off, z, a_log, dskip, states, taps, raw, positions, cu_q, slots, state,
+                   out, num_seqs) -> None:
+    """The selective scan over the step's tokens; out = y * silu(z).  dt float32 [n, inner]; x, z,
+    raw rows of the compute dtype (views are fine); bc float32 rows with B at b_off and C at c_off."""
+    n, inner = dt.shape
+    for name, t in (("z", z), ("raw", raw), ("bc", bc)):
+        _rows(t, f"selective_scan {name}")
+    if dt.dtype != torch.float32 or bc.dtype != torch.float32 or not dt.is_contiguous() or not x.is_contiguous() \
+            or not out.is_contiguous() or tuple(x.shape) != (n, inner) or tuple(out.shape) != (n, inner) \
+            or x.dtype != out.dtype or z.dtype != out.dtype or raw.dtype != out.dtype \
+            or z.shape[1] < inner or raw.shape[1] < inner:
+        raise KernelError("selective_scan: mismatched shapes or dtypes")
+    if a_log.dtype != torch.float32 or tuple(a_log.shape) != (inner, states) or not a_log.is_contiguous() \
+            or dskip.dtype != torch.float32 or dskip.numel() != inner:
+        raise KernelError("selective_scan: a_log float32 [inner, states], dskip float32 [inner]")
+    _state2d(state, "selective_scan")
+    if cu_q.shape[0] < num_seqs + 1 or slots.shape[0] < num_seqs:
+        raise KernelError("selective_scan: cu_q / slots are shorter than the step's sequences")
+    check(load().shk_selective_scan(
+        _dev(dt, "dt"), _dev(x, "x"), _dev(bc, "bc"), bc.stride(0), b_off, c_off, _dev(z, "z"), z.stride(0),
+        _dev(a_log, "a_log"), _dev(dskip, "dskip"), inner, states, taps, _dev(raw, "raw"), raw.stride(0),
+        _dev(positions, "positions", torch.int32), _dev(cu_q, "cu_q", torch.int32), _dev(slots, "slots", torch.int32),
+        _dev(state, "state"), state.stride(0), _dev(out, "out"), dtype_code(out.dtype), num_seqs, _stream()))
+
+
+def rotate_half_rows(x, off, heads, dim, rot_dim, inv_freq, positions, mult: float = 1.0) -> None:
+    """Turns the pairs (i, i + rot_dim / 2) of every head at columns off + h * dim of float32 rows,
+    in place, by positions[t] * inv_freq[i], and multiplies the head by mult."""
+    _rows(x, "rotate_half_rows x")
+    if x.dtype != torch.float32:
+        raise KernelError("rotate_half_rows: float32 rows")
+    if rot_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() < rot_dim // 2):
+        raise KernelError("rotate_half_rows: inv_freq must hold rot_dim / 2 float32 values")
+    check(load().shk_rotate_half_rows(_dev(x, "x"), x.stride(0), off, heads, dim, rot_dim,
+                                      None if not rot_dim else _dev(inv_freq, "inv_freq"),
+                                      _dev(positions, "positions", torch.int32), float(mult), x.shape[0], _stream()))
+
+
+def retention_state_floats(heads: int, dim: int, v_dim: int) -> int:
+    return int(load().shk_retention_state_floats(heads, dim, v_dim))
+
+
+def retention_scan(proj, q_off, k_off, v_off, decay, num_seqs, heads, dim, v_dim, positions, cu_q, slots, state,
+                   out) -> None:
+    """S_t = decay S_(t-1) + k v^T, o = S^T q per head over the step's tokens; proj float32 rows,
+    out float32 [n, heads * v_dim]."""
+    _rows(proj, "retention_scan proj")
+    n = proj.shape[0]
+    if proj.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (n, heads * v_dim) \
+            or not out.is_contiguous():
+        raise KernelError("retention_scan: proj and out must be float32, out contiguous [n, heads * v_dim]")
+    if decay.dtype != torch.float32 or decay.numel() != heads:
+        raise KernelError("retention_scan: one float32 decay per head")
+    _state2d(state, "retention_scan")
+    if cu_q.shape[0] < num_seqs + 1 or slots.shape[0] < num_seqs:
+        raise KernelError("retention_scan: cu_q / slots are shorter than the step's sequences")
+    check(load().shk_retention_scan(
+        _dev(proj, "proj"), proj.stride(0), q_off, k_off, v_off, _dev(decay, "decay"), num_seqs, heads, dim, v_dim,
+        _dev(positions, "positions", torch.int32), _dev(cu_q, "cu_q", torch.int32), _dev(slots, "slots", torch.int32),
+        _dev(state, "state"), state.stride(0), _dev(out, "out"), _stream()))
+
+
+def moe_route(logits, correction, top: int, chosen, weights) -> None:
+    """softmax over float32 logits [n, experts]; the `top` largest of score + correction chosen
+    (int32 [n, top]), weights their scores over the chosen ones' sum (float32 [n, top])."""
+    _rows(logits, "moe_route logits")
+    n, experts = logits.shape
+    if logits.dtype != torch.float32 or chosen.dtype != torch.int32 or weights.dtype != torch.float32 \
+            or tuple(chosen.shape) != (n, top) or tuple(weights.shape) != (n, top) \
+            or not chosen.is_contiguous() or not weights.is_contiguous():
+        raise KernelError("moe_route: logits float32 [n, experts], chosen int32 / weights float32 [n, top]")
+    if correction is not None and (correction.dtype != torch.float32 or correction.numel() != experts):
+        raise KernelError("moe_route: one float32 correction per expert")
+    check(load().shk_moe_route(_dev(logits, "logits"), logits.stride(0),
+                               None if correction is None else _dev(correction, "correction"), experts, top,
+                               _dev(chosen, "chosen"), _dev(weights, "weights"), n, _stream()))
+
+
+def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activation: str = "silu", add=None) -> None:
+    """out = add + sum_k weights[:, k] * down_e(act(gate_e x) * up_e x), e = chosen[:, k]; matrices
+    stacked [experts, ff, width] / [experts, width, ff] row-major in x's dtype."""
+    n, width = x.shape
+    experts, ff, _ = w_gate.shape
+    top = chosen.shape[1]
+    tensors = (x, w_gate, w_up, w_down, act_buf, out) + (() if add is None else (add,))
+    if any(t.dtype != x.dtype or not t.is_contiguous() for t in tensors):
+        raise KernelError("moe_experts: tensors must be contiguous and of one dtype")
+    if tuple(w_gate.shape) != (experts, ff, width) or tuple(w_up.shape) != (experts, ff, width) \
+            or tuple(w_down.shape) != (experts, width, ff) or tuple(out.shape) != (n, width) \
+            or act_buf.numel() < n * top * ff or (add is not None and tuple(add.shape) != (n, width)) \
+            or tuple(weights.shape) != (n, top) or chosen.dtype != torch.int32 or weights.dtype != torch.float32:
+        raise KernelError("moe_experts: mismatched shapes")
+    check(load().shk_moe_experts(_dev(x, "x"), _dev(chosen, "chosen"), _dev(weights, "weights"), _dev(w_gate, "w_gate"),
+                                 _dev(w_up, "w_up"), _dev(w_down, "w_down"), None if add is None else _dev(add, "add"),
+                                 _dev(act_buf, "act_buf"), _dev(out, "out"), dtype_code(x.dtype), n, width, ff, experts,
+                                 top, activation_code(activation), _stream()))
 
 
 def xielu(x, out, a_pos: float, a_neg: float) -> None:

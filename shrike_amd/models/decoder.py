@@ -7,7 +7,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelSpec
-from ..parts.base import HiddenState, ParamSpec, Part, StateSpec, build_part
+from ..parts.base import CompositeSpec, HiddenState, ParamSpec, Part, StateSpec, build_part
 
 
 class DecoderModel:
@@ -31,6 +31,9 @@ class DecoderModel:
         # some run adds the embedding's output to the stream again: it is kept
         self._keep_embedding = any(e.add_embedding for e in spec.schedule)
         self.stream_vectors: dict = {}
+        # every run's result is kept and the stream that goes on is a weighted sum of them
+        self._averaged = bool(spec.schedule) and spec.schedule[0].depth_average is not None
+        self.depth_coefficients: list = []
         # the parts whose prepare() does something, in the order they run
         self._preparers = [p for p in self.parts() if type(p).prepare is not Part.prepare]
 
@@ -50,6 +53,9 @@ class DecoderModel:
             out += block.params()
         out += [ParamSpec(name, (rows, self.spec.hidden_size), init="vector", keep_float32=True)
                 for name, rows in self.spec.stream_vectors]
+        if self._averaged:
+            out += [ParamSpec(entry.depth_average, (pos + 2,), init="average", keep_float32=True)
+                    for pos, entry in enumerate(self.spec.schedule)]
         return out + self.final_norm.params() + self.head.params()
 
     def graph_safe(self) -> bool:
@@ -61,7 +67,9 @@ class DecoderModel:
                 return False
         for block in self.blocks:
             mixer = block.mixer
-            if isinstance(mixer.cache_spec(), StateSpec) and not mixer.state_graph_safe:
+            need = mixer.cache_spec()
+            needs = [s for _, s in need.parts] if isinstance(need, CompositeSpec) else [need]
+            if any(isinstance(s, StateSpec) for s in needs) and not mixer.state_graph_safe:
                 return False
         if self.embedding_state is not None and not getattr(self.embedding, "state_graph_safe", False):
             return False
@@ -93,6 +101,9 @@ class DecoderModel:
             block.check(runtime)
             block.load(tensors, runtime)
         self.stream_vectors = {name: tensors[name] for name, _rows in self.spec.stream_vectors}
+        if self._averaged:
+            self.depth_coefficients = [tensors[e.depth_average].contiguous() for e in self.spec.schedule]
+            self._one = torch.ones(1, dtype=torch.float32, device=runtime.device)
         self.final_norm.load(tensors, runtime)
         self.head.check(runtime)
         self.head.load(tensors, runtime)
@@ -113,7 +124,21 @@ class DecoderModel:
         else:
             hidden = HiddenState(self.embedding.forward(ctx))
         embedded = self.embedding.forward(ctx, into="embedded") if self._keep_embedding else None
+        history = None
+        if self._averaged:
+            # slot 0: the embedding's output; slot k + 1: run k's working stream, which starts as
+            # the average that run k - 1 left and ends as run k's result; the last slot: what
+            # goes on to the final norm
+            from ..kernels import ops
+
+            runs = len(self.spec.schedule)
+            history = ctx.buffer("stream_history", (runs + 2, ctx.num_tokens, self.spec.hidden_size), torch.float32)
+            first = hidden.resid.view(1, ctx.num_tokens, self.spec.hidden_size)
+            ops.mix_history(first, self._one, 1, history[0])
+            ops.mix_history(first, self._one, 1, history[1])
         for pos, entry in enumerate(self.spec.schedule):
+            if history is not None:
+                hidden = HiddenState(history[pos + 1])
             if entry.add_embedding or entry.add_vector is not None:
                 from ..kernels import ops
 
@@ -123,6 +148,18 @@ class DecoderModel:
                     vector = self.stream_vectors[entry.add_vector[0]][entry.add_vector[1]]
                 ops.add_rows(hidden.resid, embedded if entry.add_embedding else None, vector)
             self.blocks[entry.block].forward(ctx, hidden, caches[pos])
+            if history is not None:
+                # the run's result is its stream plus what is pending; a pending output with a
+                # layer norm of its own is normed and added by the averaging kernel itself
+                norm = hidden.pending_norm
+                if hidden.pending is not None and not (norm is not None and len(norm) == 3):
+                    hidden.settle(ctx)
+                ops.mix_history(history, self.depth_coefficients[pos], pos + 2, history[pos + 2],
+                                delta=hidden.pending, dnorm=norm if hidden.pending is not None else None,
+                                dtype=ctx.dtype)
+                hidden.pending = hidden.pending_norm = None
+        if history is not None:
+            hidden = HiddenState(history[len(self.spec.schedule) + 1])
         rows = ctx.out_rows
         if rows.shape[0] == 0:
             return ctx.buffer("logits", (0, self.spec.vocab_size), torch.float32)

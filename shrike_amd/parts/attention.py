@@ -168,7 +168,15 @@ class PagedAttention(Mixer):
         s = self.spec
         return bool(self.value_dim != s.head_dim or getattr(s, "query_temperature", None)
                     or getattr(s, "value_norm_eps", None) or getattr(s, "softcap", None)
-                    or getattr(s, "sinks", False))
+                    or getattr(s, "sinks", False) or self.talking)
+
+    @property
+    def talking(self) -> bool:
+        """Whether the step's attention runs in the kernels that keep a token's heads together:
+        a distance bias, a sink of fixed score, or weights mixed across heads."""
+        s = self.spec
+        return bool(getattr(s, "distance_bias", False) or getattr(s, "fixed_sink", None) is not None
+                    or getattr(s, "talking_heads", False))
 
     def params(self):
         s, h = self.spec, self.width
@@ -180,6 +188,11 @@ class PagedAttention(Mixer):
         out.append(ParamSpec(t("o"), (h, s.num_heads * self.value_dim)))
         if getattr(s, "sinks", False):
             out.append(ParamSpec(t("sink"), (s.num_heads,), init="bias", keep_float32=True))
+        if getattr(s, "distance_bias", False):
+            out += [ParamSpec(t("r1"), (s.num_heads,), init="positive", keep_float32=True),
+                    ParamSpec(t("r2"), (s.num_heads,), init="positive", keep_float32=True)]
+        if getattr(s, "talking_heads", False):
+            out.append(ParamSpec(t("talk"), (s.num_heads, s.num_heads), init="near_identity", keep_float32=True))
         if s.qkv_bias:
             out += [ParamSpec(t(f"{r}_bias"), (q if r == "q" else kv,), init="bias", keep_float32=True)
                     for r in ("q", "k") + (() if s.values_from_keys else ("v",))]
@@ -189,7 +202,7 @@ class PagedAttention(Mixer):
 
     _DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-                      "o_bias": "o_proj.bias", "sink": "sinks"}
+                      "o_bias": "o_proj.bias", "sink": "sinks", "r1": "r1", "r2": "r2", "talk": "talk"}
 
     def _tensor(self, role: str) -> str:
         return self.tensor_name(role, self._DEFAULT_NAMES[role])
@@ -213,6 +226,10 @@ class PagedAttention(Mixer):
                 raise ValueError(f"{self.name}: query_temperature must be (coef, every) with every >= 1, got {qt}")
             if getattr(s, "softcap", None) is not None and not s.softcap > 0:
                 raise ValueError(f"{self.name}: softcap must be positive, got {s.softcap}")
+        if self.talking and (getattr(s, "sinks", False) or getattr(s, "softcap", None)
+                             or getattr(s, "query_temperature", None) or getattr(s, "value_norm_eps", None)):
+            raise ValueError(f"{self.name}: a distance bias, a fixed sink and mixed heads are built without "
+                             "learned sinks, capped scores, a query temperature and normed values")
         if s.num_heads % s.num_kv_heads:
             raise ValueError(
                 f"{self.name}: {s.num_heads} query heads are not a multiple of "
@@ -237,6 +254,10 @@ class PagedAttention(Mixer):
         self.w_o = runtime.weight(tensors[t("o")])
         self.b_o = tensors[t("o_bias")] if s.out_bias else None
         self.sinks = tensors[t("sink")].contiguous() if getattr(s, "sinks", False) else None
+        bias = getattr(s, "distance_bias", False)
+        self.r1 = tensors[t("r1")].contiguous() if bias else None
+        self.r2 = tensors[t("r2")].contiguous() if bias else None
+        self.talk = tensors[t("talk")].contiguous() if getattr(s, "talking_heads", False) else None
         if self.position is not None:
             self.position.load(tensors, runtime)
         self.linear = runtime.linear
@@ -248,7 +269,8 @@ class PagedAttention(Mixer):
     @property
     def plan_key(self):
         s = self.spec
-        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window, s.chunk, self.plain_store)
+        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window, s.chunk, self.plain_store,
+                self.talking)
 
     def prepare(self, shape) -> None:
         """Decides once per step and head geometry how attention is launched:
@@ -260,6 +282,15 @@ class PagedAttention(Mixer):
         s = self.spec
         h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
         plan = shape.notes[key] = AttentionPlan()
+        if self.talking:
+            # a token's heads stay together in one workgroup; single tokens with many keys share
+            # them among workgroups (bfloat16 only: float32 keeps one order of summation whatever
+            # the step holds)
+            reach = min(x for x in (s.window, s.chunk, _pow2(shape.max_decode_ctx or 1, KEYS_PER_WORKGROUP)) if x)
+            if self.dtype == torch.bfloat16 and shape.num_decode == shape.num_seqs and shape.num_decode:
+                plan.nsplit = max(1, min(compute_units() // _pow2(shape.num_decode), -(-reach // 256), 32))
+            shape.launch_key.append((key, "talking", plan.nsplit))
+            return
         plan.mfma = self.dtype == torch.bfloat16 and self.value_dim == d and ops.attention_supports_mfma(
             h, hkv, d, shape.page_size, self._qkv_width())
         # capped scores and sinks are built into the decode kernel and the shared-key prompt
@@ -322,6 +353,14 @@ class PagedAttention(Mixer):
             raise RuntimeError(f"{self.name}: the step was not prepared for this mixer "
                                "(the step function calls prepare() on every part)")
         q = qkv[:, : h * d]
+        if self.talking:
+            floats = ops.attention_talking_scratch_floats(q.shape[0], h, self.value_dim, plan.nsplit)
+            scratch = ctx.buffer("attn_talking_scratch", (floats,), torch.float32)
+            ops.attention_talking(q, out, h, hkv, d, self.value_dim, ctx.positions, ctx.token_seq, tables,
+                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale, scratch,
+                                  chunk=s.chunk, r1=self.r1, r2=self.r2, talk=self.talk,
+                                  sink=getattr(s, "fixed_sink", None), nshare=plan.nsplit)
+            return
         if not plan.mfma:
             ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.pools["k"],
                           cache.pools["v"], cache.page_size, s.window, s.scale, chunk=s.chunk,

@@ -119,12 +119,30 @@ class StateSpec:
     dtype: str = "float32"
 
 
+@dataclass(frozen=True)
+class CompositeSpec:
+    """Cache need of a mixer that is made of several mixers: ((sub-name, PagedSpec |
+    StateSpec), ...), one entry for each of them that keeps something.  The mixer gets a
+    LayerCache whose `parts[sub-name]` is the LayerCache of that entry."""
+
+    parts: tuple
+
+    def __post_init__(self):
+        names = [name for name, _ in self.parts]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a composite cache needs entries with distinct names, got {names}")
+        if any(not isinstance(spec, (PagedSpec, StateSpec)) for _, spec in self.parts):
+            raise TypeError("the entries of a composite cache are PagedSpec or StateSpec")
+
+
 class HiddenState:
     """The residual stream of a step: `resid` float32 [N, width], plus a part's
     output `pending` (compute dtype, or the partial sums of a split product) that
     has not been added yet.  The next norm adds it while it reads the row anyway.
     `pending_norm` = (weight float32 [width], eps) says that `pending` joins the
-    stream as pending * rsqrt(mean(pending^2) + eps) * weight, row by row."""
+    stream as pending * rsqrt(mean(pending^2) + eps) * weight, row by row;
+    (weight, bias, eps) that it joins as its layer norm, (pending - mean) /
+    sqrt(var + eps) * weight + bias."""
 
     __slots__ = ("resid", "pending", "pending_norm")
 
@@ -139,7 +157,9 @@ class HiddenState:
 
         if self.pending is None:
             return
-        if self.pending_norm is not None:
+        if self.pending_norm is not None and len(self.pending_norm) == 3:
+            ops.add_layernorm(self.resid, self.pending, dnorm=self.pending_norm, dtype=ctx.dtype)
+        elif self.pending_norm is not None:
             weight, eps = self.pending_norm
             ops.add_normed_rmsnorm(self.resid, self.pending, weight, eps, dtype=ctx.dtype)
         else:

@@ -101,3 +101,62 @@ class ParallelResidualBlock(Block):
 
 
 register_block("parallel_residual", ParallelResidualBlock)
+
+
+class SandwichResidualBlock(Block):
+    """x += post(mixer(pre(x))); x += post'(ffn(pre'(x))): a norm before and after each
+    sublayer.  Nothing is added here: a sublayer's output stays pending together with the
+    norm that brings it to the stream, and the next kernel that reads the stream (the next
+    norm, or whatever follows the block) norms and adds it in the same pass."""
+
+    def __init__(self, spec, width, name):
+        super().__init__(spec, width, name)
+        self.mixer_norm = build_part("norm", spec.mixer_norm, width, f"{name}.{spec.mixer_norm_name}")
+        self.mixer = build_part("mixer", spec.mixer, width, f"{name}.{spec.mixer_name}")
+        self.mixer_post = build_part("norm", spec.mixer_post, width, f"{name}.{spec.mixer_post_name}")
+        self.ffn_norm = self.ffn = self.ffn_post = None
+        if spec.ffn is not None:
+            self.ffn_norm = build_part("norm", spec.ffn_norm, width, f"{name}.{spec.ffn_norm_name}")
+            self.ffn = build_part("ffn", spec.ffn, width, f"{name}.{spec.ffn_name}")
+            self.ffn_post = build_part("norm", spec.ffn_post, width, f"{name}.{spec.ffn_post_name}")
+        listed = (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post)
+        self.parts = tuple(p for p in listed if p is not None) + tuple(getattr(self.mixer, "parts", ()))
+
+    def params(self):
+        own = (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post)
+        return [p for part in own if part is not None for p in part.params()]
+
+    def check(self, runtime):
+        for part in (self.mixer_post, self.ffn_post):
+            if part is not None and not hasattr(part, "as_pending"):
+                raise ValueError(f"{self.name}: the norm after a sublayer must be one that a pending output "
+                                 "can carry (layernorm)")
+        for part in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post):
+            if part is not None:
+                part.check(runtime)
+
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for part in self.parts)
+
+    @property
+    def launches_follow_shape(self):
+        return all(part.launches_follow_shape for part in self.parts)
+
+    def load(self, tensors, runtime):
+        for part in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post):
+            if part is not None:
+                part.load(tensors, runtime)
+
+    def forward(self, ctx, hidden: HiddenState, cache) -> None:
+        x = self.mixer_norm.forward(ctx, hidden)
+        hidden.pending = self.mixer.forward(ctx, x, cache)
+        hidden.pending_norm = self.mixer_post.as_pending()
+        if self.ffn is None:
+            return
+        x = self.ffn_norm.forward(ctx, hidden)
+        hidden.pending = self.ffn.forward(ctx, x)
+        hidden.pending_norm = self.ffn_post.as_pending()
+
+
+register_block("sandwich_residual", SandwichResidualBlock)

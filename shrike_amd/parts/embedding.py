@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import Embedding, ParamSpec, StateSpec, register_embedding
+from .base import Embedding, ParamSpec, StateSpec, build_part, register_embedding
 
 
 class TokenEmbedding(Embedding):
@@ -14,18 +14,34 @@ class TokenEmbedding(Embedding):
 
     launches_follow_shape = True
 
+    def __init__(self, spec, width, name):
+        super().__init__(spec, width, name)
+        norm = getattr(spec, "norm", None)
+        # a norm that the looked-up rows pass before they become the stream
+        self.norm = build_part("norm", norm, width, spec.norm_name) if norm is not None else None
+
     def params(self):
-        return [ParamSpec(self.tensor_name("weight"), (self.spec.vocab_size, self.width), init="embedding")]
+        own = [ParamSpec(self.tensor_name("weight"), (self.spec.vocab_size, self.width), init="embedding")]
+        return own + (self.norm.params() if self.norm is not None else [])
+
+    def check(self, runtime):
+        if self.norm is not None and not hasattr(self.norm, "normalize_"):
+            raise ValueError(f"{self.name}: the embedding's norm must be one that norms float32 rows in place "
+                             "(layernorm)")
 
     def load(self, tensors, runtime):
         self.table = tensors[self.tensor_name("weight")]
         self.scale = float(getattr(self.spec, "scale", 1.0))
+        if self.norm is not None:
+            self.norm.load(tensors, runtime)
 
     def forward(self, ctx, into: str = "resid") -> torch.Tensor:
         """Into the workspace buffer `into`; a model that needs the embedding's output
         again later asks for it a second time under another name."""
         resid = ctx.buffer(into, (ctx.num_tokens, self.width), torch.float32)
         ops.embed(self.table, ctx.token_ids, resid, self.scale)
+        if self.norm is not None:
+            self.norm.normalize_(resid)
         return resid
 
 

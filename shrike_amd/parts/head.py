@@ -9,7 +9,8 @@ from .base import Head, ParamSpec, register_head
 
 class LinearHead(Head):
     """logits = x @ W.T without bias, float32 out (reference:
-    shrike/models/qwen.py:178,192).  When the model ties its weights and the
+    shrike/models/qwen.py:178,192); by the spec also multiplied by a scale and then
+    capped, cap * tanh(logits / cap).  When the model ties its weights and the
     file carries no output matrix, W is the embedding table itself
     (qwen.py:211-212)."""
 
@@ -40,6 +41,11 @@ class LinearHead(Head):
         logits = ctx.buffer("logits", (x.shape[0], self.spec.vocab_size), torch.float32)
         if x.shape[0]:
             self.linear(x, self.weight, logits)
+            scale, cap = float(getattr(self.spec, "scale", 1.0)), getattr(self.spec, "softcap", None)
+            if scale != 1.0 or cap:
+                from ..kernels import ops
+
+                ops.scale_softcap(logits, scale, cap)
         return logits
 
 

@@ -3,7 +3,8 @@ written out as a model folder (config.json, model.safetensors) that the
 ordinary loader reads back.
 
 Matrices and biases are N(0, 0.02), norm weights 1 + N(0, 0.1) ("norm_zero", a
-norm weight stored around zero: N(0, 0.1)).  Every tensor
+norm weight stored around zero: N(0, 0.1)); the kinds that some mixers need are
+listed with their spreads below.  Every tensor
 has a generator of its own, seeded from the seed and the tensor's name, so a
 tensor's values do not depend on which other tensors exist.
 """
@@ -20,7 +21,10 @@ from safetensors.torch import save_file
 
 from ..parts.base import ParamSpec
 
-_STD = {"matrix": 0.02, "embedding": 0.02, "bias": 0.02, "norm": 0.1, "norm_zero": 0.1, "vector": 0.02}
+_STD = {"matrix": 0.02, "embedding": 0.02, "bias": 0.02, "norm": 0.1, "norm_zero": 0.1, "vector": 0.02,
+        # numbers that must be positive (|N(0, 0.5)| + 0.01), logarithms of rates, a square matrix
+        # near the identity, and coefficients of an average (1 / count + N(0, 0.05))
+        "positive": 0.5, "log_rate": 0.5, "near_identity": 0.1, "average": 0.05}
 
 #: "reference": the distributions above.  "unit": matrices N(0, 1/fan_in) (the
 #: embedding table N(0, 1)), biases N(0, 0.1): every part's output is as large
@@ -48,11 +52,19 @@ def random_tensor(p: ParamSpec, seed: int, dtype: torch.dtype, device="cpu",
             std = 1.0
         elif p.init in ("bias", "vector"):
             std = 0.1
+        elif p.init == "average":
+            std = 0.2
     elif mode != "reference":
         raise ValueError(f"init mode must be one of {INIT_MODES}, got {mode!r}")
     t = torch.empty(p.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
     if p.init == "norm":
         t += 1.0
+    elif p.init == "positive":
+        t = t.abs() + 0.01
+    elif p.init == "near_identity":
+        t += torch.eye(p.shape[0], p.shape[1], device=device)
+    elif p.init == "average":
+        t += 1.0 / p.shape[0]
     return t.to(dtype)
 
 
