@@ -637,7 +637,7 @@ __global__ void __launch_bounds__(GM* GN* kWave)
     for (int i = 0; i < kAPer; ++i) {
       const int rb = (wave + kWaves * i) / KS;
       const int token = tok0 + rb * 16 + lane % 16;
-      asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (lane / 16) * 8;
+      asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda;  // + (lane / 16) * 8 where that lies in the row
     }
     // Two named sets of registers, not an array of two: an array indexed by the
     // loop's step would live in scratch memory.
@@ -645,8 +645,9 @@ __global__ void __launch_bounds__(GM* GN* kWave)
     auto fetch = [&](u32x4 (&hw)[kWPer], u32x4 (&hx)[kAPer], int st) {
 #pragma unroll
       for (int i = 0; i < kAPer; ++i) {
-        const int col = (st * KS + (wave + kWaves * i) % KS) * 32;  // + (lane / 16) * 8 in asrc
-        hx[i] = *reinterpret_cast<const u32x4*>(asrc[i] + (col + (lane / 16) * 8 < k ? col : 0));
+        // (columns beyond k: the row's first 16 bytes, numbers that meet the weight tiles' zeros)
+        const int col = (st * KS + (wave + kWaves * i) % KS) * 32 + (lane / 16) * 8;
+        hx[i] = *reinterpret_cast<const u32x4*>(asrc[i] + (col < k ? col : 0));
       }
 #pragma unroll
       for (int i = 0; i < kWPer; ++i) {
@@ -786,17 +787,17 @@ __global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per
   for (int i = 0; i < kAPer; ++i) {
     const int f = wave + kWaves * i;
     const int token = kUnits ? tok0 + (f / 2) * 16 + (f % 2) * 8 + lane % 8 : tok0 + (f / KS) * 16 + lane % 16;
-    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (kUnits ? lane / 8 : lane / 16) * 8;
+    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda;  // + the lane's chunk where it lies in the row
   }
   const int xunit = (lane % 16) / 8, xplace = lane % 8 + 8 * (lane / 16);
   auto load = [&](u32x4 (&buf)[kFrags][kWave], int st) {
     const int stage = st < all_stages ? st : 0;  // past the end: any stage, never multiplied
 #pragma unroll
     for (int i = 0; i < kAPer; ++i) {
-      // (+ the lane's chunk, which is in asrc)
-      const int col = kUnits ? stage * 64 : (stage * KS + (wave + kWaves * i) % KS) * 32;
-      SHK_LOAD_TO_LDS(asrc[i] + (col + (kUnits ? lane / 8 : lane / 16) * 8 < k ? col : 0),
-                      &buf[kWFrags + wave + kWaves * i][0]);
+      // (a chunk beyond k: the row's first 16 bytes, numbers that meet the weight tiles' zeros)
+      const int col = (kUnits ? stage * 64 : (stage * KS + (wave + kWaves * i) % KS) * 32) +
+                      (kUnits ? lane / 8 : lane / 16) * 8;
+      SHK_LOAD_TO_LDS(asrc[i] + (col < k ? col : 0), &buf[kWFrags + wave + kWaves * i][0]);
     }
 #pragma unroll
     for (int i = 0; i < kWPer; ++i) {
@@ -950,7 +951,7 @@ __global__ void __launch_bounds__(16 * kWave)
     f = f < kFrags ? f : f % kFrags;
     afrag[i] = f;
     const int token = (f / KT) * 16 + (f % 2) * 8 + lane % 8;
-    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (lane / 8) * 8;
+    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda;  // + (lane / 8) * 8 where that lies in the row
   }
   auto fetch = [&](u32x4 (&buf)[kFrags][kWave], u32x4 (&w)[KT], int st) {
     // past the share's end: some stage that exists, never multiplied
@@ -958,8 +959,10 @@ __global__ void __launch_bounds__(16 * kWave)
     stage = stage < 0 ? 0 : stage;
 #pragma unroll
     for (int i = 0; i < APER; ++i) {
-      const int col = (stage * KT + ((afrag[i] % KT) / 2) * 2) * 32;  // + (lane / 8) * 8 in asrc
-      SHK_LOAD_TO_LDS(asrc[i] + (col + (lane / 8) * 8 < k ? col : 0), &buf[afrag[i]][0]);
+      // a chunk beyond k is fetched from the row's first 16 bytes instead (it meets zeros of the
+      // weight tiles' padding, so it must be numbers, not whatever lies behind the matrix)
+      const int col = (stage * KT + ((afrag[i] % KT) / 2) * 2) * 32 + (lane / 8) * 8;
+      SHK_LOAD_TO_LDS(asrc[i] + (col < k ? col : 0), &buf[afrag[i]][0]);
     }
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
