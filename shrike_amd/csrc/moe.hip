@@ -71,6 +71,22 @@ __global__ void __launch_bounds__(256)
         best_e = oe;
       }
     }
+    if (best_e >= experts) {
+      // no score compares (logits that are not numbers): the lowest expert not yet taken, so
+      // that what is written is always an expert's index
+      best_e = 1 << 30;
+#pragma unroll
+      for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+        const int e = lane + i * kWave;
+        if (e < experts && !(c[i] == -INFINITY) && e < best_e) best_e = e;
+      }
+#pragma unroll
+      for (int off = kWave / 2; off > 0; off >>= 1) {
+        const int oe = __shfl_xor(best_e, off, kWave);
+        best_e = oe < best_e ? oe : best_e;
+      }
+      if (best_e >= experts) best_e = k;  // (cannot happen while top <= experts)
+    }
     float score = 0.f;
 #pragma unroll
     for (int i = 0; i < kMaxExpertsPerLane; ++i) {
@@ -102,10 +118,11 @@ constexpr int kMoeFeatures = 32;  // features (or columns) a workgroup
 template <typename T>
 __global__ void __launch_bounds__(256)
     moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ chosen, const T* __restrict__ wg,
-                       const T* __restrict__ wu, T* __restrict__ act_out, int width, int ff, int top, int act) {
+                       const T* __restrict__ wu, T* __restrict__ act_out, int width, int ff, int top, int act,
+                       int experts) {
   extern __shared__ float xs[];
   const int pair = blockIdx.y, t = pair / top;
-  const int e = chosen[pair];
+  const int e = min(max(chosen[pair], 0), experts - 1);  // an index from memory never leaves the stack of experts
   for (int k = threadIdx.x; k < width; k += 256) xs[k] = to_float(x[static_cast<size_t>(t) * width + k]);
   __syncthreads();
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -129,7 +146,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
     moe_down_kernel(const T* __restrict__ act_in, const int32_t* __restrict__ chosen,
                     const float* __restrict__ weights, const T* __restrict__ wd, const T* __restrict__ add,
-                    T* __restrict__ out, int width, int ff, int top) {
+                    T* __restrict__ out, int width, int ff, int top, int experts) {
   extern __shared__ float as[];  // [top, ff]
   const int t = blockIdx.y;
   for (int i = threadIdx.x; i < top * ff; i += 256) as[i] = to_float(act_in[static_cast<size_t>(t) * top * ff + i]);
@@ -140,7 +157,7 @@ __global__ void __launch_bounds__(256)
     if (c >= width) break;
     float total = 0.f;
     for (int k = 0; k < top; ++k) {
-      const int e = chosen[static_cast<size_t>(t) * top + k];
+      const int e = min(max(chosen[static_cast<size_t>(t) * top + k], 0), experts - 1);
       const T* dr = wd + (static_cast<size_t>(e) * width + c) * ff;
       float d = 0.f;
       for (int f = lane; f < ff; f += kWave) d = fmaf(to_float(dr[f]), as[k * ff + f], d);
@@ -189,10 +206,10 @@ extern "C" int shk_moe_experts(const void* x, const int32_t* chosen, const float
   moe_gate_up_kernel<T><<<g1, 256, width * sizeof(float), s>>>(static_cast<const T*>(x), chosen,                      \
                                                                static_cast<const T*>(w_gate),                         \
                                                                static_cast<const T*>(w_up), static_cast<T*>(act_buf), \
-                                                               width, ff, top, act);                                  \
+                                                               width, ff, top, act, experts);                         \
   moe_down_kernel<T><<<g2, 256, static_cast<size_t>(top) * ff * sizeof(float), s>>>(                                  \
       static_cast<const T*>(act_buf), chosen, weights, static_cast<const T*>(w_down), static_cast<const T*>(add),     \
-      static_cast<T*>(out), width, ff, top)
+      static_cast<T*>(out), width, ff, top, experts)
   if (dtype == kF32) {
     SHK_GO(float);
   } else {

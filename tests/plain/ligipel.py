@@ -61,6 +61,28 @@ def sink_softmax(s: torch.Tensor, visible: torch.Tensor) -> torch.Tensor:
     return e / (torch.exp(-m) + e.sum(dim=-1, keepdim=True))
 
 
+def mixed_head_attention(q, k, v, scale: float, window, r1, r2, talk, sink: bool = True):
+    """q [n, H, D], k [n, G, D], v [n, G, V] -> [n, H, V]: scores less the distance bias, a
+    sliding window (None: all earlier keys), the softmax with a sink of score 0, the weights
+    mixed across heads by talk [H, H], each head on the values of its own key/value head."""
+    n, H, _ = q.shape
+    G, V = k.shape[1], v.shape[2]
+    visible = window_mask(n, window if window is not None else n + 1)
+    bias = distance_bias(n, r1, r2) if r1 is not None else torch.zeros(H, n, n, dtype=q.dtype)
+    p = torch.zeros(H, n, n, dtype=q.dtype)
+    for head in range(H):
+        s = (q[:, head] @ k[:, head // (H // G)].T) * scale - bias[head]
+        if sink:
+            p[head] = sink_softmax(s, visible)
+        else:
+            p[head] = torch.softmax(s.masked_fill(~visible, float("-inf")), dim=-1)
+    mixed = torch.einsum("hg,gij->hij", talk, p) if talk is not None else p
+    out = torch.zeros(n, H, V, dtype=q.dtype)
+    for head in range(H):
+        out[:, head] = mixed[head] @ v[:, head // (H // G)]
+    return out
+
+
 def talking_attention(h, w, prefix: str, m: dict):
     """Grouped-query attention without rotation: a logarithmic distance bias, a sliding
     window, a sink of score 0, and weights mixed across heads after the softmax."""
@@ -69,17 +91,9 @@ def talking_attention(h, w, prefix: str, m: dict):
     q = (h @ w[prefix + ".q"].T).view(n, H, D)
     k = (h @ w[prefix + ".k"].T).view(n, G, D)
     v = (h @ w[prefix + ".v"].T).view(n, G, V)
-    visible = window_mask(n, int(m["mask"]["size"]))
-    bias = distance_bias(n, w[prefix + ".r1"].to(h.dtype), w[prefix + ".r2"].to(h.dtype))
-    p = torch.zeros(H, n, n, dtype=h.dtype)
-    for head in range(H):
-        g = head // (H // G)
-        s = (q[:, head] @ k[:, g].T) * float(m["scale"]) - bias[head]
-        p[head] = sink_softmax(s, visible)
-    mixed = torch.einsum("hg,gij->hij", w[prefix + ".talk"].to(h.dtype), p)
-    out = torch.zeros(n, H, V, dtype=h.dtype)
-    for head in range(H):
-        out[:, head] = mixed[head] @ v[:, head // (H // G)]
+    window = int(m["mask"]["size"]) if m.get("mask") else None
+    out = mixed_head_attention(q, k, v, float(m["scale"]), window, w[prefix + ".r1"].to(h.dtype),
+                               w[prefix + ".r2"].to(h.dtype), w[prefix + ".talk"].to(h.dtype))
     return out.reshape(n, H * V) @ w[prefix + ".o"].T
 
 
@@ -95,10 +109,21 @@ def causal_conv(x, taps, bias):
     return y
 
 
+def scan(x, dt, A, B, C, D, S=None):
+    """x, dt [n, inner]; A [inner, N]; B, C [n, N]; D [inner] -> (y [n, inner], final S):
+    S <- exp(dt A) S + dt x B^T per token; y = S C + D x."""
+    n, inner = x.shape
+    S = torch.zeros(inner, A.shape[1], dtype=x.dtype) if S is None else S.clone()
+    y = torch.zeros(n, inner, dtype=x.dtype)
+    for t in range(n):
+        S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
+        y[t] = S @ C[t] + D * x[t]
+    return y, S
+
+
 def selective_scan(h, w, prefix: str, m: dict):
     """Mamba: a per-channel linear recurrence whose step size and input/output maps
     depend on the token."""
-    n = h.shape[0]
     inner, R, N = m["inner"], m["dt_rank"], m["state"]
     xz = h @ w[prefix + ".in"].T
     x, z = xz[:, :inner], xz[:, inner:]
@@ -107,12 +132,7 @@ def selective_scan(h, w, prefix: str, m: dict):
     dt, B, C = dbc[:, :R], dbc[:, R : R + N], dbc[:, R + N :]
     dt = F.softplus(dt @ w[prefix + ".dt"].T + w[prefix + ".dt.b"].to(h.dtype))  # [n, inner]
     A = -torch.exp(w[prefix + ".A_log"].to(h.dtype))  # [inner, N]
-    D = w[prefix + ".D"].to(h.dtype)
-    S = torch.zeros(inner, N, dtype=h.dtype)
-    y = torch.zeros(n, inner, dtype=h.dtype)
-    for t in range(n):
-        S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
-        y[t] = S @ C[t] + D * x[t]
+    y, _ = scan(x, dt, A, B, C, w[prefix + ".D"].to(h.dtype))
     return (y * silu(z)) @ w[prefix + ".o"].T
 
 
@@ -136,9 +156,23 @@ def rotate_half(x, positions, dims: int, base: float):
     return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., dims:]], dim=-1)
 
 
+def retention(q, k, v, decay, S=None):
+    """q, k [n, H, D], v [n, H, V] -> (o [n, H, V], final S [H, D, V]):
+    S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t."""
+    n, H, D = q.shape
+    V = v.shape[2]
+    S = torch.zeros(H, D, V, dtype=q.dtype) if S is None else S.clone()
+    o = torch.zeros(n, H, V, dtype=q.dtype)
+    for t in range(n):
+        for head in range(H):
+            S[head] = float(decay[head]) * S[head] + k[t, head][:, None] * v[t, head][None, :]
+            o[t, head] = S[head].T @ q[t, head]
+    return o, S
+
+
 def retention_mixer(h, positions, w, prefix: str, m: dict, eps: float):
-    """Linear attention with a fixed decay per head: S_t = decay S_(t-1) + k_t v_t^T,
-    o_t = S_t^T q_t; no softmax, no denominator."""
+    """Linear attention with a fixed decay per head, no softmax, no denominator; the
+    readout normed per head, gated and projected."""
     n = h.shape[0]
     H, D, V = m["heads"], m["dim"], m["vdim"]
     rot = m.get("rot") or {}
@@ -146,12 +180,7 @@ def retention_mixer(h, positions, w, prefix: str, m: dict, eps: float):
     q = rotate_half((h @ w[prefix + ".q"].T).view(n, H, D), positions, dims, base)
     k = rotate_half((h @ w[prefix + ".k"].T).view(n, H, D), positions, dims, base) * D**-0.5
     v = (h @ w[prefix + ".v"].T).view(n, H, V)
-    o = torch.zeros(n, H, V, dtype=h.dtype)
-    for head in range(H):
-        S = torch.zeros(D, V, dtype=h.dtype)
-        for t in range(n):
-            S = float(m["decay"][head]) * S + k[t, head][:, None] * v[t, head][None, :]
-            o[t, head] = S.T @ q[t, head]
+    o, _ = retention(q, k, v, m["decay"])
     o = unit_rms(o, eps).reshape(n, H * V)
     return (o * silu(h @ w[prefix + ".g"].T)) @ w[prefix + ".o"].T
 
@@ -214,7 +243,38 @@ def forward(cfg: dict, w: dict, tokens, keep_layers: bool = False):
         x = sum(coef[j] * history[j] for j in range(i + 2))
         kept.append(x)
     x = layer_norm(x, w["final.norm"].to(x.dtype), w["final.norm.b"].to(x.dtype), eps)
-    logits = (x @ w["head"].T) * float(cfg["logit_scale"])
-    cap = float(cfg["logit_softcap"])
-    logits = cap * torch.tanh(logits / cap)
+    logits = (x @ w["head"].T) * float(cfg.get("logit_scale", 1.0))
+    if cfg.get("logit_softcap"):
+        cap = float(cfg["logit_softcap"])
+        logits = cap * torch.tanh(logits / cap)
     return (logits, torch.stack(kept)) if keep_layers else logits
+
+
+class PlainLigipel:
+    """A model folder read once; `logits(ids)`, the stream after every layer, and greedy
+    generation over it, in float64 unless told otherwise."""
+
+    def __init__(self, model_dir, dtype=torch.float64):
+        import json
+        from pathlib import Path
+
+        from safetensors.torch import load_file
+
+        self.cfg = json.loads((Path(model_dir) / "config.json").read_text())
+        raw = load_file(str(Path(model_dir) / "model.safetensors"))
+        self.weights = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in raw.items()}
+
+    def logits(self, token_ids, rows=None) -> torch.Tensor:
+        out = forward(self.cfg, self.weights, list(token_ids))
+        return out if rows is None else out[torch.tensor(list(rows), dtype=torch.long)]
+
+    def layers(self, token_ids) -> torch.Tensor:
+        return forward(self.cfg, self.weights, list(token_ids), keep_layers=True)[1]
+
+    def greedy(self, prompt, max_new_tokens: int) -> list[int]:
+        seq, out = list(prompt), []
+        for _ in range(max_new_tokens):
+            tok = int(torch.argmax(self.logits(seq)[-1]))
+            out.append(tok)
+            seq.append(tok)
+        return out
