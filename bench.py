@@ -76,7 +76,8 @@ def prefill_flops(cfg, n: int) -> float:
     layers, head = matmul_params(cfg)
     linear = 2.0 * n * layers + 2.0 * head  # the output matrix runs on one row
     # causal attention: token p reads p + 1 keys, 2 products of head_dim each per head
-    attn = 4.0 * cfg.head_dim * cfg.num_attention_heads * cfg.num_hidden_layers * n * (n + 1) / 2
+    attn_layers = getattr(cfg, "attention_layers", cfg.num_hidden_layers)
+    attn = 4.0 * cfg.head_dim * cfg.num_attention_heads * attn_layers * n * (n + 1) / 2
     return linear + attn
 
 
@@ -170,7 +171,9 @@ def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int,
         engine.abort(req.req_id)
     layer_w, head_w = matmul_params(cfg)
     mean_ctx = (context_start + context_end) / 2 + 1
-    step_bytes = 2.0 * (layer_w + head_w) + batch * mean_ctx * kv_bytes_per_token(cfg)
+    # (a design with recurrent layers reads and writes each request's state once a step)
+    step_bytes = (2.0 * (layer_w + head_w) + batch * mean_ctx * kv_bytes_per_token(cfg)
+                  + batch * getattr(cfg, "state_bytes_per_seq", 0))
     ms = elapsed / steps * 1e3
     return {
         "tok_s": produced / elapsed, "ms_per_step": ms, "context_start": context_start,
@@ -323,7 +326,9 @@ def kernel_breakdown(engine, steps: int = 3, before_step=None) -> dict:
              "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample",
              "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows", "embed_pairs", "qkv_store",
              "latent_prepare", "rotate_heads", "latent_attention", "latent_attention_mfma", "gemm_batched", "mlstm_scan", "headnorm_gate",
-             "xielu"]
+             "xielu", "layernorm", "add_layernorm", "attention_talking", "conv_silu", "dt_softplus", "selective_scan",
+             "rotate_half_rows", "retention_scan", "moe_route", "moe_experts", "mix_history", "scale_softcap"]
+    names = [n for n in names if hasattr(ops, n)]
     spans: list[tuple[str, object, object]] = []
     saved = {n: getattr(ops, n) for n in names}
 
@@ -447,6 +452,64 @@ def minilorn_like(qcfg, window: int, pattern: str):
     return mcfg, sizes
 
 
+def ligipel_like(qcfg, window: int, pattern: str, experts: int, top: int):
+    """A Ligipel configuration with the layer sizes of a Qwen2 one (same width, vocabulary and
+    number of layers).  `pattern` says which mixer each layer has, letter by letter, repeated:
+    p, attention with Qwen2's heads (sliding window `window`) beside a selective scan of
+    `width` channels with 16 states, 4 taps and a step-size rank of width / 16; r, retention
+    with width / 256 heads of 128 query/key and 256 value elements.  Every layer has `experts`
+    routed experts of which a token uses `top`, and a shared one half as wide as Qwen2's
+    feed-forward; the chosen experts together are the other half.  With it an object that
+    names the sizes as the formulas of this program expect them; its `at_batch(b)` sets the
+    matrices' elements that a step of b tokens reads (the experts that b tokens are expected
+    to touch when the router spreads them evenly)."""
+    from types import SimpleNamespace
+
+    from shrike_amd.models.ligipel import (BiasedAttention, DecayedRetention, LigipelConfig, LigipelLayer, Mixture,
+                                           Scan, SideBySide)
+
+    h, d, H, KV = qcfg.hidden_size, qcfg.head_dim, qcfg.num_attention_heads, qcfg.num_key_value_heads
+    inter = qcfg.intermediate_size
+    ff = max(64, inter // (2 * top) // 64 * 64)
+    shared = inter // 2
+    scan = Scan(inner=h, state=16, dt_rank=max(1, h // 16), conv=4)
+    rheads = max(1, h // 256)
+    mixers = {
+        "p": ("parallel", SideBySide(left=BiasedAttention(heads=H, kv_heads=KV, dim=d, vdim=d, scale=d**-0.5,
+                                                          window=window), right=scan)),
+        "r": ("retention", DecayedRetention(heads=rheads, dim=128, vdim=256,
+                                            decay=tuple(1.0 - 2.0 ** (-5 - i % 8) for i in range(rheads)),
+                                            rot_base=10000.0, rot_dims=64)),
+    }
+    kinds = [mixers[pattern[i % len(pattern)]] for i in range(qcfg.num_hidden_layers)]
+    mlp = Mixture(experts=experts, top=top, ff=ff, shared_ff=shared)
+    lcfg = LigipelConfig(vocab=qcfg.vocab_size, width=h, norm_eps=qcfg.rms_norm_eps,
+                         layers=tuple(LigipelLayer(kind, mixer, mlp) for kind, mixer in kinds),
+                         logit_scale=1.0, logit_softcap=30.0)
+    n = len(kinds)
+    elements = {
+        "parallel": 2 * (H + KV) * d * h + 3 * scan.inner * h + (scan.dt_rank + 2 * scan.state) * scan.inner
+        + scan.inner * scan.dt_rank * 2,  # (the step-size matrix is float32)
+        "retention": (2 * rheads * 128 + 3 * rheads * 256) * h,
+    }
+    states = {"parallel": scan.inner * (scan.state + scan.conv - 1), "retention": rheads * 128 * 256}
+    mixer_elements = sum(elements[k] for k, _ in kinds) // n
+    sizes = SimpleNamespace(
+        hidden_size=h, head_dim=d, num_attention_heads=H, num_key_value_heads=KV, intermediate_size=inter,
+        num_hidden_layers=n, vocab_size=qcfg.vocab_size, attention_layers=sum(k == "parallel" for k, _ in kinds),
+        kv_elements_per_token=sum(2 * KV * d for k, _ in kinds if k == "parallel"),
+        state_bytes_per_seq=2 * 4 * sum(states[k] for k, _ in kinds))
+
+    def at_batch(b: int) -> None:
+        touched = experts * (1.0 - (1.0 - top / experts) ** b)
+        sizes.layer_elements = int(mixer_elements + experts * h + 3 * h * shared + touched * 3 * h * ff)
+
+    sizes.at_batch = at_batch
+    # a prompt: every token's own experts are work, whichever matrices hold them
+    sizes.layer_elements = mixer_elements + experts * h + 3 * h * shared + top * 3 * h * ff
+    return lcfg, sizes
+
+
 def run_designs(args, qcfg) -> dict:
     """Another design beside Qwen2 at equal layer sizes, random weights: a prompt of 2,048
     tokens in one step, decode steps at batch 1, 8 and 64 from that context, and what each
@@ -456,9 +519,13 @@ def run_designs(args, qcfg) -> dict:
     import torch
 
     from shrike_amd import SamplingParams
-    from shrike_amd.models import minilorn, mofarax, qwen2
+    from shrike_amd.models import ligipel, minilorn, mofarax, qwen2
 
-    if args.minilorn:
+    if args.ligipel:
+        lcfg, lsizes = ligipel_like(qcfg, args.window, args.pattern if set(args.pattern) <= set("pr") else "pppr",
+                                    args.experts, args.top)
+        other = ("ligipel", ligipel.build_spec(lcfg), lsizes)
+    elif args.minilorn:
         mcfg, msizes = minilorn_like(qcfg, args.window, args.pattern)
         other = ("minilorn", minilorn.build_spec(mcfg), msizes)
     else:
@@ -478,6 +545,8 @@ def run_designs(args, qcfg) -> dict:
         res = {"prefill": run_prefill(engine, sizes, args.seed)}
         res["prefill_kernels_us"] = kernel_breakdown(engine, steps=2, before_step=add_prompt)
         for batch in (1, 8, 64):
+            if hasattr(sizes, "at_batch"):
+                sizes.at_batch(batch)
             d = run_decode(engine, sizes, batch, args.design_steps, args.warmup, args.seed)
             res[f"decode_b{batch}"] = {"tok_s": round(d["tok_s"], 1), "ms_per_step": round(d["ms_per_step"], 3),
                                        "roofline_frac": round(d["gb_s"] / HBM_PEAK_GBS, 3)}
@@ -640,12 +709,17 @@ def main() -> int:
                          "--shape, random weights: prompt, decode at batch 1 / 8 / 64, per-kernel times")
     ap.add_argument("--minilorn", action="store_true",
                     help="Minilorn beside Qwen2 at equal layer sizes: prompt, decode at batch 1/8/64, time per kernel")
+    ap.add_argument("--ligipel", action="store_true",
+                    help="Ligipel beside Qwen2 at equal layer sizes: prompt, decode at batch 1/8/64, time per kernel")
+    ap.add_argument("--experts", type=int, default=8, metavar="N", help="--ligipel: routed experts a layer")
+    ap.add_argument("--top", type=int, default=2, metavar="N", help="--ligipel: experts a token uses")
     ap.add_argument("--pattern", default="alml", metavar="LETTERS",
-                    help="--minilorn: the layers' mixers in order, repeated: a(ttention), l(atent attention), m(atrix memory)")
+                    help="--minilorn: the layers' mixers in order, repeated: a(ttention), l(atent attention), m(atrix memory); "
+                         "--ligipel: p(arallel attention and scan), r(etention), default pppr")
     ap.add_argument("--window", type=int, default=4096, metavar="N",
                     help="--minilorn: sliding window of its latent attention (4096: no fewer keys than Qwen2 reads)")
-    ap.add_argument("--design-only", choices=["qwen2", "mofarax", "minilorn"], default=None,
-                    help="--mofarax / --minilorn: run only this one of the two (for a profile of one model's kernels)")
+    ap.add_argument("--design-only", choices=["qwen2", "mofarax", "minilorn", "ligipel"], default=None,
+                    help="--mofarax / --minilorn / --ligipel: run only this one of the two (for a profile of one model's kernels)")
     ap.add_argument("--mask-size", type=int, default=8192, metavar="N",
                     help="--mofarax: positions per block of its attention (8192: no fewer keys than Qwen2 reads)")
     ap.add_argument("--side-dim", type=int, default=256, metavar="N", help="--mofarax: width of its per-layer token input")
@@ -678,12 +752,14 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
-    if args.mofarax or args.minilorn:
+    if args.mofarax or args.minilorn or args.ligipel:
         designs = run_designs(args, cfg)
-        design = "Minilorn" if args.minilorn else "Mofarax"
+        design = "Ligipel" if args.ligipel else "Minilorn" if args.minilorn else "Mofarax"
         config = {"shape": args.shape, "layers": cfg.num_hidden_layers, "prompt": PROMPT_LEN,
                   "decode_steps": args.design_steps}
-        config.update({"pattern": args.pattern, "window": args.window} if args.minilorn
+        config.update({"pattern": args.pattern if set(args.pattern) <= set("pr") else "pppr", "window": args.window,
+                       "experts": args.experts, "top": args.top} if args.ligipel
+                      else {"pattern": args.pattern, "window": args.window} if args.minilorn
                       else {"mask_size": args.mask_size, "side_dim": args.side_dim})
         print(json.dumps({
             "metric": f"{design} beside Qwen2 at the Qwen2.5-{args.shape.upper()} layer sizes: prompt tok/s, decode "
