@@ -313,6 +313,22 @@ int shk_attention_talking(const void* q, int q_stride, void* out, int dtype, int
                           const float* r1, const float* r2, const float* talk, int has_sink, float sink,
                           float* scratch, int nshare, void* stream);
 
+// The same for bfloat16 on the matrix units, where shk_attention_talking_supports_mfma says so:
+// every head's own weights meet the values of every key/value head (one pass over the keys with a
+// running maximum and sum), and the sums are mixed: o_h = sum_g talk[h, g] U[g, c(h)].  The step's
+// first num_single tokens are single tokens of sequences 0 .. num_single - 1; prompt portions come
+// as num_tiles tiles of 16 queries (tile_seq, tile_q0 counted from the portion's first query; cu_q[s]
+// = sequence s's first row).  scratch: shk_attention_talking_mfma_scratch_floats(...) floats.
+int shk_attention_talking_supports_mfma(int head_dim, int v_dim, int page_size, int q_stride);
+long long shk_attention_talking_mfma_scratch_floats(int n, int heads, int kv_heads, int v_dim);
+int shk_attention_talking_bf16(const void* q, int q_stride, void* out, int n, int num_single, int num_tiles,
+                               int heads, int kv_heads, int head_dim, int v_dim, const int32_t* positions,
+                               const int32_t* token_seq, const int32_t* cu_q, const int32_t* tile_seq,
+                               const int32_t* tile_q0, const int32_t* tables, int table_stride, const void* k_pool,
+                               const void* v_pool, int page_size, int num_pages, int window, int chunk, float scale,
+                               const float* r1, const float* r2, const float* talk, int has_sink, float sink,
+                               float* scratch, void* stream);
+
 // The selective scan of Mamba and its causal convolution (ssm.hip).  A request's slot holds S
 // [inner, states] float32 and then the convolution's last taps - 1 inputs [(taps - 1), inner].
 // shk_conv_silu: y[t, c] = silu(bias[c] + sum_k taps[c, num_taps - 1 - k] * x[t - k, c]) over the
@@ -357,6 +373,13 @@ int shk_moe_route(const float* logits, int ld, const float* correction, int expe
 int shk_moe_experts(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
                     const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
                     int dtype, int n, int width, int ff, int experts, int top, int act, void* stream);
+// The same for bfloat16 on the matrix units, expert by expert over the lists of the (token,
+// expert) pairs that chose it (built on the device).  width and ff in multiples of 8; scratch:
+// shk_moe_grouped_scratch_bytes(...) bytes, 16-byte aligned.
+long long shk_moe_grouped_scratch_bytes(int n, int width, int experts, int top);
+int shk_moe_experts_grouped(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
+                            const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
+                            void* scratch, int n, int width, int ff, int experts, int top, int act, void* stream);
 
 // out = a_pos z^2 + z / 2 where z > 0, a_neg (exp(z) - 1 - z) + z / 2 elsewhere; elementwise.
 int shk_xielu(const void* x, void* out, int dtype, long long numel, float a_pos, float a_neg, void* stream);
@@ -407,7 +430,7 @@ long long shk_sample_scratch_floats(int rows, int vocab);
 // `stream` is passed instead.  The calls run in order on `stream`; the first that
 // refuses its arguments ends the run with its status and message (those before it
 // have been launched).
-#define SHK_CALL_MAX_ARGS 28
+#define SHK_CALL_MAX_ARGS 32
 typedef struct shk_call {
   int32_t launcher;
   int32_t reserved;

@@ -206,6 +206,238 @@ __global__ void __launch_bounds__(256)
   out[static_cast<size_t>(t) * outs + o] = from_float<T>(sum);
 }
 
+// ---------------------------------------------------------------- bfloat16 on the matrix units
+//
+// Mixing the weights of a key across heads and then summing the values is the same as summing
+// the values with every head's own weights and mixing the sums:
+//
+//   o_h = sum_j (sum_g talk[h, g] p_g(j)) v_c(j) = sum_g talk[h, g] U[g, c],   c = h's key/value head,
+//   U[g, c] = sum_j p_g(j) v_c(j)
+//
+// so each softmax head g runs as ordinary attention with a running maximum and sum, only
+// that its weights meet the values of every key/value head, and a small kernel mixes the
+// results.  One pass over the keys, no weights in memory.
+//
+// A wavefront serves 16 query rows that share a sequence and a key/value head for the keys:
+// 16 consecutive tokens of a prompt's portion for one head (tile_seq / tile_q0 list them), or
+// one single token's heads of a key/value head.  Keys go by in chunks of 32, aligned to 32 in
+// the sequence:
+//
+//   S^T = K Q^T   [32 keys x 16 rows]  two v_mfma_f32_16x16x32_bf16 per 32 elements of a head;
+//                 A = keys straight from their slabs (a lane's 8 elements are 16 bytes), and
+//                 the keys are assigned to A's rows so that a lane ends up with the scores of
+//                 8 consecutive keys of its query row: P^T is then already a B operand
+//   softmax       base 2, float32, running maximum and sum per row (lanes i, i+16, i+32, i+48)
+//   O^T += V^T P^T  [16 values x 16 rows] per block of 16 value elements and key/value head;
+//                 A = 8 consecutive keys of one value element, 16 bytes of the transposed pool
+//
+// NB: blocks of 16 value elements that a pass holds (value heads of a pass x blocks a head);
+// KS: 32-element steps of a head.  Value heads beyond a pass are other workgroups (grid z),
+// which form the scores again.
+typedef __bf16 tbf16x8 __attribute__((ext_vector_type(8)));
+typedef float tf32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float rows_max(float v) {  // over lanes i, i + 16, i + 32, i + 48
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  return fmaxf(v, __shfl_xor(v, 32, kWave));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  v += __shfl_xor(v, 16, kWave);
+  return v + __shfl_xor(v, 32, kWave);
+}
+
+template <int KS, int NB>
+__global__ void __launch_bounds__(256)
+    talking_mfma_kernel(const bf16* __restrict__ q, int q_stride, float* __restrict__ u_out, int heads, int kv_heads,
+                        int head_dim, int v_dim, const int32_t* __restrict__ positions,
+                        const int32_t* __restrict__ token_seq, const int32_t* __restrict__ tables, int table_stride,
+                        const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool, int page_size, int num_pages,
+                        int window, int chunk, float scale_l2, const float* __restrict__ r1,
+                        const float* __restrict__ r2, int has_sink, float sink_l2, const int32_t* __restrict__ cu_q,
+                        const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int tiles_mode,
+                        int first_token, int vh_pass) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int i = lane % 16, kg = lane / 16;
+  const int group = heads / kv_heads;
+  const int unit = blockIdx.y * 4 + wave;
+  const int vb = (v_dim + 15) / 16;  // blocks of 16 value elements a head
+  const int cv0 = blockIdx.z * vh_pass;
+  const int cvn = min(vh_pass, kv_heads - cv0);
+  // the lane's query row
+  int t, head, seq, ck;
+  bool valid;
+  if (tiles_mode) {
+    if (unit >= heads) return;
+    seq = tile_seq[blockIdx.x];
+    t = cu_q[seq] + tile_q0[blockIdx.x] + i;
+    valid = t < cu_q[seq + 1];
+    head = unit;
+    ck = head / group;
+  } else {
+    const int subs = (group + 15) / 16;
+    if (unit >= kv_heads * subs) return;
+    t = first_token + blockIdx.x;
+    seq = token_seq[t];
+    ck = unit / subs;
+    const int within = (unit % subs) * 16 + i;
+    valid = within < group;
+    head = ck * group + (valid ? within : 0);
+  }
+  const int pos = valid ? positions[t] : -1;
+  const int lo = valid ? first_key(pos, window, chunk) : (1 << 30);
+  int pos_max = pos, lo_min = lo;
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) {
+    pos_max = max(pos_max, __shfl_xor(pos_max, off, kWave));
+    lo_min = min(lo_min, __shfl_xor(lo_min, off, kWave));
+  }
+  if (pos_max < 0) return;  // (no row of the tile is a token)
+  const int32_t* table = tables + static_cast<size_t>(seq) * table_stride;
+  const float bias1 = r1 ? r1[head] : 0.f, bias2 = r1 ? r2[head] : 0.f;
+  // the queries: B operands, elements ks * 32 + kg * 8 .. + 8 of row i
+  tbf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    const int e = ks * 32 + kg * 8;
+    if (valid && e < head_dim)
+      v = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(t) * q_stride + head * head_dim + e);
+    qf[ks] = __builtin_bit_cast(tbf16x8, v);
+  }
+  tf32x4 o[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) o[b] = tf32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = has_sink ? sink_l2 : -INFINITY;
+  float l_run = has_sink ? 1.f : 0.f;
+  const int slab = key_slab(head_dim);
+  const size_t k_head = static_cast<size_t>(page_size) * head_dim;  // elements of a page's head
+  const size_t v_head = static_cast<size_t>(page_size) * v_dim;
+  for (int j0 = lo_min / 32 * 32; j0 <= pos_max; j0 += 32) {
+    // scores: A row m of product t2 is the key j0 + 8 (m / 4) + 4 t2 + m % 4
+    tf32x4 s[2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      s[t2] = tf32x4{0.f, 0.f, 0.f, 0.f};
+      const int jk = j0 + 8 * (i / 4) + 4 * t2 + i % 4;
+      int page = -1;
+      if (jk >= lo_min && jk <= pos_max) {
+        page = table[jk / page_size];
+        if (page < 0 || page >= num_pages) page = -1;
+      }
+      const bf16* kr = k_pool + (static_cast<size_t>(max(page, 0)) * kv_heads + ck) * k_head;
+      const int slot = jk % page_size;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        uint4 kv = make_uint4(0, 0, 0, 0);
+        const int e = ks * 32 + kg * 8;
+        if (page >= 0 && e < head_dim)
+          kv = *reinterpret_cast<const uint4*>(kr + (static_cast<size_t>(e / slab) * page_size + slot) * slab + e % slab);
+        s[t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, kv), qf[ks], s[t2], 0, 0, 0);
+      }
+    }
+    // this lane: the scores of keys j0 + 8 kg + 4 t2 + r for its row i; their page (8 aligned keys share one)
+    const int jg = j0 + 8 * kg;
+    int vpage = -1;
+    if (jg + 7 >= lo_min && jg <= pos_max) {
+      vpage = table[jg / page_size];
+      if (vpage < 0 || vpage >= num_pages) vpage = -1;
+    }
+    float x[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int j = jg + 4 * t2 + r;
+        float v = s[t2][r] * scale_l2;
+        if (r1) v -= bias1 * __log2f(1.f + bias2 * static_cast<float>(pos - j));
+        const bool seen = vpage >= 0 && j >= lo && j <= pos;
+        v = seen ? v : -INFINITY;
+        x[4 * t2 + r] = v;
+        mx = fmaxf(mx, v);
+      }
+    const float m_new = fmaxf(m_run, rows_max(mx));
+    const float alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_new) : 0.f;
+    float psum = 0.f;
+    union {
+      uint4 u;
+      uint16_t h[8];
+    } pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float p = x[e] > -INFINITY ? __builtin_amdgcn_exp2f(x[e] - m_new) : 0.f;
+      psum += p;
+      const bf16 pb = from_float<bf16>(p);
+      pf.h[e] = __builtin_bit_cast(uint16_t, pb);
+    }
+    l_run = l_run * alpha + rows_sum(psum);
+    m_run = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[b][r] *= alpha;
+    }
+    // values: A row i of block b is value element (b % vb) * 16 + i of key/value head cv0 + b / vb, keys jg .. + 8
+    const int slot = jg % page_size;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int cvl = b / vb, d = (b % vb) * 16 + i;
+      union {
+        uint4 u;
+        uint16_t h[8];
+      } vf;
+      vf.u = make_uint4(0, 0, 0, 0);
+      if (cvl < cvn) {
+        if (vpage >= 0 && d < v_dim) {
+          vf.u = *reinterpret_cast<const uint4*>(v_pool + (static_cast<size_t>(vpage) * kv_heads + cv0 + cvl) * v_head +
+                                                 static_cast<size_t>(d) * page_size + slot);
+          if (jg < lo_min || jg + 7 > pos_max) {  // keys that no row of the tile reads may hold anything
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (jg + e < lo_min || jg + e > pos_max) vf.h[e] = 0;
+          }
+        }
+        o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, vf.u), __builtin_bit_cast(tbf16x8, pf.u),
+                                                       o[b], 0, 0, 0);
+      }
+    }
+  }
+  if (!valid) return;
+  // this lane holds value elements (b % vb) * 16 + 4 kg + r of its row
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  float* dst = u_out + (static_cast<size_t>(t) * heads + head) * kv_heads * v_dim;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int cvl = b / vb;
+    if (cvl >= cvn) continue;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int d = (b % vb) * 16 + 4 * kg + r;
+      if (d < v_dim) dst[static_cast<size_t>(cv0 + cvl) * v_dim + d] = o[b][r] * inv;
+    }
+  }
+}
+
+// out[t, h, d] = sum_g talk[h, g] * U[t, g, c(h), d]   (talk null: U[t, h, c(h), d])
+__global__ void __launch_bounds__(256)
+    talking_mix_kernel(const float* __restrict__ u_in, const float* __restrict__ talk, bf16* __restrict__ out, int heads,
+                       int kv_heads, int v_dim) {
+  const int t = blockIdx.y;
+  const int o = blockIdx.x * blockDim.x + threadIdx.x;
+  if (o >= heads * v_dim) return;
+  const int h = o / v_dim, d = o % v_dim;
+  const int c = h / (heads / kv_heads);
+  const float* ut = u_in + static_cast<size_t>(t) * heads * kv_heads * v_dim + static_cast<size_t>(c) * v_dim + d;
+  float sum = 0.f;
+  if (talk) {
+    for (int g = 0; g < heads; ++g) sum = fmaf(talk[h * heads + g], ut[static_cast<size_t>(g) * kv_heads * v_dim], sum);
+  } else {
+    sum = ut[static_cast<size_t>(h) * kv_heads * v_dim];
+  }
+  out[static_cast<size_t>(t) * heads * v_dim + o] = from_float<bf16>(sum);
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -265,5 +497,106 @@ extern "C" int shk_attention_talking(const void* q, int q_stride, void* out, int
   }
 #undef SHK_GO
   SHK_LAUNCH_CHECK("attention_talking");
+  return 0;
+}
+
+// bfloat16 on the matrix units.  The step's first `num_single` tokens are single tokens of their
+// sequences; the prompt portions that follow are listed in tiles of 16 queries (tile_seq, tile_q0
+// from the portion's first query; cu_q[s] is sequence s's first row).  scratch: n * heads *
+// kv_heads * v_dim floats.
+extern "C" int shk_attention_talking_supports_mfma(int head_dim, int v_dim, int page_size, int q_stride) {
+  return head_dim % 8 == 0 && head_dim <= 256 && v_dim >= 1 && v_dim <= 256 && page_size % 8 == 0 && q_stride % 8 == 0;
+}
+
+extern "C" long long shk_attention_talking_mfma_scratch_floats(int n, int heads, int kv_heads, int v_dim) {
+  return static_cast<long long>(n) * heads * kv_heads * v_dim;
+}
+
+namespace shk {
+
+template <int KS, int NB>
+static void launch_talking_mfma(dim3 grid, hipStream_t s, const bf16* q, int q_stride, float* u, int heads, int kv_heads,
+                                int head_dim, int v_dim, const int32_t* positions, const int32_t* token_seq,
+                                const int32_t* tables, int table_stride, const bf16* k_pool, const bf16* v_pool,
+                                int page_size, int num_pages, int window, int chunk, float scale_l2, const float* r1,
+                                const float* r2, int has_sink, float sink_l2, const int32_t* cu_q,
+                                const int32_t* tile_seq, const int32_t* tile_q0, int tiles_mode, int first_token,
+                                int vh_pass) {
+  talking_mfma_kernel<KS, NB><<<grid, 256, 0, s>>>(q, q_stride, u, heads, kv_heads, head_dim, v_dim, positions, token_seq,
+                                                   tables, table_stride, k_pool, v_pool, page_size, num_pages, window,
+                                                   chunk, scale_l2, r1, r2, has_sink, sink_l2, cu_q, tile_seq, tile_q0,
+                                                   tiles_mode, first_token, vh_pass);
+}
+
+}  // namespace shk
+
+extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out, int n, int num_single, int num_tiles,
+                                          int heads, int kv_heads, int head_dim, int v_dim, const int32_t* positions,
+                                          const int32_t* token_seq, const int32_t* cu_q, const int32_t* tile_seq,
+                                          const int32_t* tile_q0, const int32_t* tables, int table_stride,
+                                          const void* k_pool, const void* v_pool, int page_size, int num_pages,
+                                          int window, int chunk, float scale, const float* r1, const float* r2,
+                                          const float* talk, int has_sink, float sink, float* scratch, void* stream) {
+  SHK_REQUIRE(n >= 0 && num_single >= 0 && num_single <= n && num_tiles >= 0 && heads > 0 && kv_heads > 0 &&
+                  heads % kv_heads == 0,
+              "attention_talking_bf16: bad sizes n=%d single=%d tiles=%d heads=%d kv_heads=%d", n, num_single, num_tiles,
+              heads, kv_heads);
+  SHK_REQUIRE(shk_attention_talking_supports_mfma(head_dim, v_dim, page_size, q_stride),
+              "attention_talking_bf16: head_dim %d, v_dim %d, page_size %d or q_stride %d is not served", head_dim, v_dim,
+              page_size, q_stride);
+  SHK_REQUIRE(q_stride >= heads * head_dim && page_size > 0 && num_pages > 0 && table_stride > 0,
+              "attention_talking_bf16: bad strides or cache sizes");
+  SHK_REQUIRE(static_cast<int64_t>(num_pages) * kv_heads * page_size < (1LL << 31),
+              "attention_talking_bf16: cache pool has too many rows for 32-bit row indices");
+  SHK_REQUIRE((r1 == nullptr) == (r2 == nullptr), "attention_talking_bf16: the distance bias needs both of its numbers");
+  if (n == 0) return 0;
+  SHK_REQUIRE(q && out && positions && token_seq && tables && k_pool && v_pool && scratch,
+              "attention_talking_bf16: null pointer");
+  SHK_REQUIRE(num_tiles == 0 || (cu_q && tile_seq && tile_q0), "attention_talking_bf16: tiles without their lists");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pool) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(v_pool) % 16 == 0,
+              "attention_talking_bf16: operands must be 16-byte aligned");
+  SHK_REQUIRE(n <= 65535 && num_tiles <= 0x7fffffff / 4, "attention_talking_bf16: at most 65535 tokens a call, got %d", n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float log2e = 1.4426950408889634f;
+  const int ks = (head_dim + 31) / 32, vb = (v_dim + 15) / 16;
+  const int group = heads / kv_heads;
+#define SHK_GO(KS, NB)                                                                                                 \
+  launch_talking_mfma<KS, NB>(grid, s, static_cast<const bf16*>(q), q_stride, scratch, heads, kv_heads, head_dim, v_dim, \
+                              positions, token_seq, tables, table_stride, static_cast<const bf16*>(k_pool),             \
+                              static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale * log2e, r1,  \
+                              r2, has_sink, sink * log2e, cu_q, tile_seq, tile_q0, mode, 0, vh_pass)
+#define SHK_NB(KS)                                                                                                     \
+  if (nb <= 2) SHK_GO(KS, 2);                                                                                          \
+  else if (nb <= 4) SHK_GO(KS, 4);                                                                                     \
+  else if (nb <= 8) SHK_GO(KS, 8);                                                                                     \
+  else if (nb <= 16) SHK_GO(KS, 16);                                                                                   \
+  else SHK_GO(KS, 32)
+#define SHK_KS()                                                                                                       \
+  if (ks <= 1) { SHK_NB(1); }                                                                                          \
+  else if (ks <= 2) { SHK_NB(2); }                                                                                     \
+  else if (ks <= 4) { SHK_NB(4); }                                                                                     \
+  else { SHK_NB(8); }
+  if (num_single > 0) {
+    // single tokens: a key/value head's query heads are a tile's rows; one value head a workgroup
+    const int mode = 0, vh_pass = 1, nb = vb;
+    const int units = kv_heads * ((group + 15) / 16);
+    dim3 grid(num_single, (units + 3) / 4, kv_heads);
+    SHK_KS()
+  }
+  if (num_tiles > 0) {
+    const int mode = 1;
+    const int vh_pass = max(1, min(kv_heads, 32 / vb));
+    const int nb = vh_pass * vb;
+    dim3 grid(num_tiles, (heads + 3) / 4, (kv_heads + vh_pass - 1) / vh_pass);
+    SHK_KS()
+  }
+#undef SHK_KS
+#undef SHK_NB
+#undef SHK_GO
+  const int outs = heads * v_dim;
+  talking_mix_kernel<<<dim3((outs + 255) / 256, n), 256, 0, s>>>(scratch, talk, static_cast<bf16*>(out), heads, kv_heads,
+                                                                v_dim);
+  SHK_LAUNCH_CHECK("attention_talking_bf16");
   return 0;
 }

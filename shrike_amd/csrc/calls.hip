@@ -84,6 +84,7 @@ const Launcher kLaunchers[] = {
     SHK_LAUNCHER(shk_mix_history),
     SHK_LAUNCHER(shk_scale_softcap),
     SHK_LAUNCHER(shk_attention_talking),
+    SHK_LAUNCHER(shk_attention_talking_bf16),
     SHK_LAUNCHER(shk_conv_silu),
     SHK_LAUNCHER(shk_dt_softplus),
     SHK_LAUNCHER(shk_selective_scan),
@@ -91,6 +92,7 @@ const Launcher kLaunchers[] = {
     SHK_LAUNCHER(shk_retention_scan),
     SHK_LAUNCHER(shk_moe_route),
     SHK_LAUNCHER(shk_moe_experts),
+    SHK_LAUNCHER(shk_moe_experts_grouped),
     SHK_LAUNCHER(shk_embed_pairs),
     SHK_LAUNCHER(shk_argmax),
     SHK_LAUNCHER(shk_sample),

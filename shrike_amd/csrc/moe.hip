@@ -12,6 +12,14 @@
 //                      order, so a token's result does not depend on what else is in the step
 // moe_down_kernel      a workgroup per (token, block of columns): the chosen experts'
 //                      outputs, weighted and added in the order they were chosen
+//
+// On the matrix units (bfloat16, many tokens): the (token, expert) pairs are listed per expert
+// in the order of the tokens (moe_lists_kernel, a workgroup per expert), and the two products
+// run per expert over its list in tiles of 32 pairs (v_mfma_f32_16x16x32_bf16, both operands
+// row-major with k innermost and loaded as operands straight from memory).  Workgroups beyond
+// an expert's list leave at once, so the grid depends on the step's size alone.  A pair's
+// sums run over k in one fixed order wherever the pair stands in its list; the pairs' outputs
+// are kept in float32 and joined per token in the order the experts were chosen.
 #include "api.h"
 #include "common.h"
 
@@ -170,6 +178,196 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+typedef __bf16 mbf16x8 __attribute__((ext_vector_type(8)));
+typedef float mf32x4 __attribute__((ext_vector_type(4)));
+
+// order[e * n + r] = the r-th pair (token * top + place among the token's choices) of expert e,
+// tokens ascending; counts[e] = how many there are
+__global__ void __launch_bounds__(256)
+    moe_lists_kernel(const int32_t* __restrict__ chosen, int n, int top, int32_t* __restrict__ order,
+                     int32_t* __restrict__ counts) {
+  __shared__ int wave_total[256 / kWave];
+  const int e = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  int base = 0;
+  for (int t0 = 0; t0 < n; t0 += 256) {
+    const int t = t0 + threadIdx.x;
+    int hit = -1;
+    if (t < n)
+      for (int k = top - 1; k >= 0; --k)
+        if (chosen[static_cast<size_t>(t) * top + k] == e) hit = k;
+    const unsigned long long votes = __ballot(hit >= 0);
+    const int before = __popcll(votes & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_total[wave] = __popcll(votes);
+    __syncthreads();
+    int prefix = 0, total = 0;
+    for (int w = 0; w < 256 / kWave; ++w) {
+      if (w < wave) prefix += wave_total[w];
+      total += wave_total[w];
+    }
+    if (hit >= 0) order[static_cast<size_t>(e) * n + base + prefix + before] = t * top + hit;
+    base += total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) counts[e] = base;
+}
+
+// act[pair, f] = act(W_gate_e[f] . x_t) * (W_up_e[f] . x_t) for the pairs of expert e's list: a workgroup
+// takes 32 pairs and four wavefronts' 32 features each
+__global__ void __launch_bounds__(256)
+    moe_gate_up_mfma_kernel(const bf16* __restrict__ x, const int32_t* __restrict__ order,
+                            const int32_t* __restrict__ counts, const bf16* __restrict__ wg,
+                            const bf16* __restrict__ wu, bf16* __restrict__ act_out, int n, int width, int ff, int top,
+                            int act) {
+  const int e = blockIdx.z;
+  const int count = min(counts[e], n);
+  const int row0 = blockIdx.y * 32;
+  if (row0 >= count) return;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int i = lane % 16, kg = lane / 16;
+  const int f0 = (blockIdx.x * 4 + wave) * 32;
+  if (f0 >= ff) return;
+  int pair[2];
+  const bf16* xr[2];
+  const bf16* gr[2];
+  const bf16* ur[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const int r = row0 + a * 16 + i;
+    pair[a] = r < count ? order[static_cast<size_t>(e) * n + r] : -1;
+    const int t = pair[a] >= 0 ? min(pair[a] / top, n - 1) : 0;
+    xr[a] = x + static_cast<size_t>(t) * width + kg * 8;
+    const int f = min(f0 + a * 16 + i, ff - 1);
+    gr[a] = wg + (static_cast<size_t>(e) * ff + f) * width + kg * 8;
+    ur[a] = wu + (static_cast<size_t>(e) * ff + f) * width + kg * 8;
+  }
+  mf32x4 accg[2][2], accu[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) accg[a][b] = accu[a][b] = mf32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < width; k0 += 32) {
+    const bool have = k0 + kg * 8 < width;  // (width is a multiple of 8: a piece is whole or absent)
+    uint4 av[2], gv[2], uv[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      av[a] = gv[a] = uv[a] = make_uint4(0, 0, 0, 0);
+      if (have) {
+        if (pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(xr[a] + k0);
+        gv[a] = *reinterpret_cast<const uint4*>(gr[a] + k0);
+        uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, gv[b]),
+                                                             __builtin_bit_cast(mbf16x8, av[a]), accg[a][b], 0, 0, 0);
+        accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
+                                                             __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
+      }
+  }
+  // features were the rows of the products: this lane holds features f0 + 16 b + 4 kg + r of pair row a * 16 + i
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    if (pair[a] < 0) continue;
+    bf16* dst = act_out + static_cast<size_t>(pair[a]) * ff;
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int f = f0 + b * 16 + 4 * kg + r;
+        if (f < ff) dst[f] = from_float<bf16>(gate_act(accg[a][b][r], act) * accu[a][b][r]);
+      }
+  }
+}
+
+// pair_out[pair, c] = W_down_e[c] . act[pair]: a workgroup takes 32 pairs and four wavefronts' 64 columns each
+__global__ void __launch_bounds__(256)
+    moe_down_mfma_kernel(const bf16* __restrict__ act_in, const int32_t* __restrict__ order,
+                         const int32_t* __restrict__ counts, const bf16* __restrict__ wd,
+                         float* __restrict__ pair_out, int n, int width, int ff, int top) {
+  const int e = blockIdx.z;
+  const int count = min(counts[e], n);
+  const int row0 = blockIdx.y * 32;
+  if (row0 >= count) return;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int i = lane % 16, kg = lane / 16;
+  const int c0 = (blockIdx.x * 4 + wave) * 64;
+  if (c0 >= width) return;
+  int pair[2];
+  const bf16* ar[2];
+  const bf16* wr[4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const int r = row0 + a * 16 + i;
+    pair[a] = r < count ? order[static_cast<size_t>(e) * n + r] : -1;
+    const int p = pair[a] >= 0 ? min(pair[a], n * top - 1) : 0;
+    ar[a] = act_in + static_cast<size_t>(p) * ff + kg * 8;
+  }
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int c = min(c0 + b * 16 + i, width - 1);
+    wr[b] = wd + (static_cast<size_t>(e) * width + c) * ff + kg * 8;
+  }
+  mf32x4 acc[2][4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = mf32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < ff; k0 += 32) {
+    const bool have = k0 + kg * 8 < ff;
+    uint4 av[2], wv[4];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      av[a] = make_uint4(0, 0, 0, 0);
+      if (have && pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(ar[a] + k0);
+    }
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      wv[b] = make_uint4(0, 0, 0, 0);
+      if (have) wv[b] = *reinterpret_cast<const uint4*>(wr[b] + k0);
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, wv[b]),
+                                                            __builtin_bit_cast(mbf16x8, av[a]), acc[a][b], 0, 0, 0);
+  }
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    if (pair[a] < 0) continue;
+    float* dst = pair_out + static_cast<size_t>(pair[a]) * width;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int c = c0 + b * 16 + 4 * kg;
+      if (c + 3 < width) {
+        *reinterpret_cast<float4*>(dst + c) = make_float4(acc[a][b][0], acc[a][b][1], acc[a][b][2], acc[a][b][3]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (c + r < width) dst[c + r] = acc[a][b][r];
+      }
+    }
+  }
+}
+
+// out[t, c] = add[t, c] + sum_k weights[t, k] * pair_out[t * top + k, c], k in the order chosen
+__global__ void __launch_bounds__(256)
+    moe_join_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, const bf16* __restrict__ add,
+                    bf16* __restrict__ out, int width, int top) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  float total = 0.f;
+  for (int k = 0; k < top; ++k)
+    total = fmaf(weights[static_cast<size_t>(t) * top + k], pair_out[(static_cast<size_t>(t) * top + k) * width + c], total);
+  if (add) total += to_float(add[static_cast<size_t>(t) * width + c]);
+  out[static_cast<size_t>(t) * width + c] = from_float<bf16>(total);
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -217,5 +415,44 @@ extern "C" int shk_moe_experts(const void* x, const int32_t* chosen, const float
   }
 #undef SHK_GO
   SHK_LAUNCH_CHECK("moe_experts");
+  return 0;
+}
+
+extern "C" long long shk_moe_grouped_scratch_bytes(int n, int width, int experts, int top) {
+  // order [experts, n] and counts [experts] (int32), then the pairs' outputs [n * top, width] (float32)
+  const long long ints = static_cast<long long>(experts) * n + experts;
+  return ((ints * 4 + 15) / 16) * 16 + static_cast<long long>(n) * top * width * 4;
+}
+
+extern "C" int shk_moe_experts_grouped(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
+                                       const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
+                                       void* scratch, int n, int width, int ff, int experts, int top, int act,
+                                       void* stream) {
+  SHK_REQUIRE(n >= 0 && width > 0 && ff > 0 && experts > 0 && experts <= 65535 && top >= 1 && top <= experts,
+              "moe_experts_grouped: bad sizes n=%d width=%d ff=%d experts=%d top=%d", n, width, ff, experts, top);
+  SHK_REQUIRE(act == 1 || act == 2, "moe_experts_grouped: unknown activation %d", act);
+  SHK_REQUIRE(width % 8 == 0 && ff % 8 == 0, "moe_experts_grouped: width %d and ff %d must be multiples of 8", width, ff);
+  if (n == 0) return 0;
+  SHK_REQUIRE(static_cast<long long>(n) * top < (1LL << 30) && (n + 31) / 32 <= 65535,
+              "moe_experts_grouped: too many (token, expert) pairs");
+  SHK_REQUIRE(x && chosen && weights && w_gate && w_up && w_down && act_buf && out && scratch,
+              "moe_experts_grouped: null pointer");
+  for (const void* p : {x, w_gate, w_up, w_down, static_cast<const void*>(act_buf), static_cast<const void*>(scratch)})
+    SHK_REQUIRE(reinterpret_cast<uintptr_t>(p) % 16 == 0, "moe_experts_grouped: operands must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* order = static_cast<int32_t*>(scratch);
+  int32_t* counts = order + static_cast<size_t>(experts) * n;
+  const long long ints = static_cast<long long>(experts) * n + experts;
+  float* pair_out = reinterpret_cast<float*>(static_cast<char*>(scratch) + ((ints * 4 + 15) / 16) * 16);
+  moe_lists_kernel<<<experts, 256, 0, s>>>(chosen, n, top, order, counts);
+  const int row_tiles = (n + 31) / 32;
+  moe_gate_up_mfma_kernel<<<dim3((ff + 127) / 128, row_tiles, experts), 256, 0, s>>>(
+      static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
+      static_cast<bf16*>(act_buf), n, width, ff, top, act);
+  moe_down_mfma_kernel<<<dim3((width + 255) / 256, row_tiles, experts), 256, 0, s>>>(
+      static_cast<const bf16*>(act_buf), order, counts, static_cast<const bf16*>(w_down), pair_out, n, width, ff, top);
+  moe_join_kernel<<<dim3((width + 255) / 256, n), 256, 0, s>>>(pair_out, weights, static_cast<const bf16*>(add),
+                                                               static_cast<bf16*>(out), width, top);
+  SHK_LAUNCH_CHECK("moe_experts_grouped");
   return 0;
 }

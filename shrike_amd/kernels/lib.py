@@ -15,7 +15,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 _LIB = None
 _RECORDING: list | None = None  # (launcher id, argument tuple) while a step is being recorded
-CALL_MAX_ARGS = 28
+CALL_MAX_ARGS = 32
 
 
 class KernelError(RuntimeError):
@@ -59,6 +59,8 @@ _SIGNATURES = {
     "shk_scale_softcap": [_P, c_longlong, _F, _F, _P],
     "shk_attention_talking": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _P, _P,
                               _P, _I, _F, _P, _I, _P],
+    "shk_attention_talking_bf16": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I,
+                                   _I, _F, _P, _P, _P, _I, _F, _P, _P],
     "shk_conv_silu": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, c_longlong, _I, _P, _I, _I, _P],
     "shk_dt_softplus": [_P, _I, _P, _P, _I, _I, _P, _I, _P],
     "shk_selective_scan": [_P, _P, _P, _I, _I, _I, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, c_longlong,
@@ -67,6 +69,7 @@ _SIGNATURES = {
     "shk_retention_scan": [_P, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, c_longlong, _P, _P],
     "shk_moe_route": [_P, _I, _P, _I, _I, _P, _P, _I, _P],
     "shk_moe_experts": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "shk_moe_experts_grouped": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_xielu": [_P, _P, _I, c_longlong, _F, _F, _P],
     "shk_embed_pairs": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],
@@ -135,10 +138,15 @@ def load():
         lib.shk_mlstm_state_floats = raw.shk_mlstm_state_floats
         for name, argtypes in (("shk_attention_talking_scratch_floats", [_I, _I, _I, _I]),
                                ("shk_selective_scan_state_floats", [_I, _I, _I]),
-                               ("shk_retention_state_floats", [_I, _I, _I])):
+                               ("shk_retention_state_floats", [_I, _I, _I]),
+                               ("shk_moe_grouped_scratch_bytes", [_I, _I, _I, _I]),
+                               ("shk_attention_talking_mfma_scratch_floats", [_I, _I, _I, _I])):
             fn = getattr(raw, name)
             fn.argtypes, fn.restype = argtypes, c_longlong
             setattr(lib, name, fn)
+        raw.shk_attention_talking_supports_mfma.argtypes = [_I, _I, _I, _I]
+        raw.shk_attention_talking_supports_mfma.restype = c_int
+        lib.shk_attention_talking_supports_mfma = raw.shk_attention_talking_supports_mfma
         raw.shk_sample_scratch_floats.argtypes = [_I, _I]
         raw.shk_sample_scratch_floats.restype = c_longlong
         lib.shk_sample_scratch_floats = raw.shk_sample_scratch_floats

@@ -777,6 +777,45 @@ def attention_talking(q, out, heads, kv_heads, head_dim, v_dim, positions, token
         _dev(scratch, "scratch"), int(nshare), _stream()))
 
 
+def attention_talking_supports_mfma(head_dim: int, v_dim: int, page_size: int, q_stride: int) -> bool:
+    return bool(load().shk_attention_talking_supports_mfma(head_dim, v_dim, page_size, q_stride))
+
+
+def attention_talking_mfma_scratch_floats(n: int, heads: int, kv_heads: int, v_dim: int) -> int:
+    return int(load().shk_attention_talking_mfma_scratch_floats(n, heads, kv_heads, v_dim))
+
+
+def attention_talking_mfma(q, out, num_single, heads, kv_heads, head_dim, v_dim, positions, token_seq, cu_q, tile_seq,
+                           tile_q0, num_tiles, tables, k_pool, v_pool, page_size, window, scale, scratch, chunk=None,
+                           r1=None, r2=None, talk=None, sink=None) -> None:
+    """attention_talking for bfloat16 on the matrix units.  The first num_single rows are single
+    tokens of sequences 0 .. num_single - 1; the prompt portions after them are listed as
+    num_tiles tiles of 16 queries (tile_seq, tile_q0: int32, q0 counted within the portion).
+    scratch: float32 of attention_talking_mfma_scratch_floats(...)."""
+    _rows(q, "attention_talking_mfma q")
+    n = q.shape[0]
+    if q.dtype != torch.bfloat16 or tuple(out.shape) != (n, heads * v_dim) or not out.is_contiguous() \
+            or out.dtype != q.dtype:
+        raise KernelError("attention_talking_mfma: bfloat16 q, out contiguous [n, heads * v_dim]")
+    for name, t, count in (("r1", r1, heads), ("r2", r2, heads), ("talk", talk, heads * heads)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != count or not t.is_contiguous()):
+            raise KernelError(f"attention_talking_mfma: {name} must be contiguous float32 of {count} values")
+    if scratch.dtype != torch.float32 or scratch.numel() < attention_talking_mfma_scratch_floats(n, heads, kv_heads, v_dim):
+        raise KernelError("attention_talking_mfma: scratch is too small")
+    if num_tiles and (tile_seq is None or tile_q0 is None or tile_seq.numel() < num_tiles or tile_q0.numel() < num_tiles):
+        raise KernelError("attention_talking_mfma: the tile lists are shorter than num_tiles")
+    _check_pools("attention_talking_mfma", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size, v_dim)
+    check(load().shk_attention_talking_bf16(
+        _dev(q, "q"), q.stride(0), _dev(out, "out"), n, num_single, num_tiles, heads, kv_heads, head_dim, v_dim,
+        _dev(positions, "positions", torch.int32), _dev(token_seq, "token_seq", torch.int32),
+        _dev(cu_q, "cu_q", torch.int32), None if not num_tiles else _dev(tile_seq, "tile_seq", torch.int32),
+        None if not num_tiles else _dev(tile_q0, "tile_q0", torch.int32), _dev(tables, "tables", torch.int32),
+        tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size, k_pool.shape[0], int(window or 0),
+        int(chunk or 0), float(scale), None if r1 is None else _dev(r1, "r1"), None if r2 is None else _dev(r2, "r2"),
+        None if talk is None else _dev(talk, "talk"), int(sink is not None), float(sink or 0.0),
+        _dev(scratch, "scratch"), _stream()))
+
+
 def selective_scan_state_floats(inner: int, states: int, taps: int) -> int:
     return int(load().shk_selective_scan_state_floats(inner, states, taps))
 
@@ -895,9 +934,24 @@ def moe_route(logits, correction, top: int, chosen, weights) -> None:
                                _dev(chosen, "chosen"), _dev(weights, "weights"), n, _stream()))
 
 
-def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activation: str = "silu", add=None) -> None:
+MOE_GROUPED_FROM = 4  # tokens of a step from which the experts' products run per expert on the matrix units
+
+
+def moe_grouped(n: int, width: int, ff: int, dtype) -> bool:
+    """Whether a step of n tokens runs its experts' products per expert on the matrix units:
+    bfloat16, rows in multiples of 8 elements, and enough tokens that experts are shared."""
+    return dtype == torch.bfloat16 and n >= MOE_GROUPED_FROM and width % 8 == 0 and ff % 8 == 0
+
+
+def moe_grouped_scratch_bytes(n: int, width: int, experts: int, top: int) -> int:
+    return int(load().shk_moe_grouped_scratch_bytes(n, width, experts, top))
+
+
+def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activation: str = "silu", add=None,
+                scratch=None) -> None:
     """out = add + sum_k weights[:, k] * down_e(act(gate_e x) * up_e x), e = chosen[:, k]; matrices
-    stacked [experts, ff, width] / [experts, width, ff] row-major in x's dtype."""
+    stacked [experts, ff, width] / [experts, width, ff] row-major in x's dtype.  scratch (uint8,
+    moe_grouped_scratch_bytes): the products run per expert on the matrix units (see moe_grouped)."""
     n, width = x.shape
     experts, ff, _ = w_gate.shape
     top = chosen.shape[1]
@@ -909,6 +963,17 @@ def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activati
             or act_buf.numel() < n * top * ff or (add is not None and tuple(add.shape) != (n, width)) \
             or tuple(weights.shape) != (n, top) or chosen.dtype != torch.int32 or weights.dtype != torch.float32:
         raise KernelError("moe_experts: mismatched shapes")
+    if scratch is not None:
+        if not moe_grouped(n, width, ff, x.dtype) or scratch.dtype != torch.uint8 \
+                or scratch.numel() < moe_grouped_scratch_bytes(n, width, experts, top):
+            raise KernelError("moe_experts: scratch is for bfloat16 steps that moe_grouped() accepts, and must hold "
+                              "moe_grouped_scratch_bytes() bytes")
+        check(load().shk_moe_experts_grouped(
+            _dev(x, "x"), _dev(chosen, "chosen"), _dev(weights, "weights"), _dev(w_gate, "w_gate"), _dev(w_up, "w_up"),
+            _dev(w_down, "w_down"), None if add is None else _dev(add, "add"), _dev(act_buf, "act_buf"),
+            _dev(out, "out"), _dev(scratch, "scratch"), n, width, ff, experts, top, activation_code(activation),
+            _stream()))
+        return
     check(load().shk_moe_experts(_dev(x, "x"), _dev(chosen, "chosen"), _dev(weights, "weights"), _dev(w_gate, "w_gate"),
                                  _dev(w_up, "w_up"), _dev(w_down, "w_down"), None if add is None else _dev(add, "add"),
                                  _dev(act_buf, "act_buf"), _dev(out, "out"), dtype_code(x.dtype), n, width, ff, experts,

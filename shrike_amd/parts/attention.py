@@ -282,6 +282,24 @@ class PagedAttention(Mixer):
         s = self.spec
         h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
         plan = shape.notes[key] = AttentionPlan()
+        if self.talking and self.dtype == torch.bfloat16 and ops.attention_talking_supports_mfma(
+                d, self.value_dim, shape.page_size, self._qkv_width()):
+            # on the matrix units: single tokens by key/value head, prompt portions in tiles of 16 queries
+            plan.kernel = "talking_mfma"
+            portions = shape.q_lens[shape.num_decode:]
+            plan.count = 0
+            if portions.size:
+                seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE)
+                keys = shape.starts[seqs] + q0  # (the heaviest tiles first)
+                order = heavy_first(np.minimum(keys, s.window) if s.window else keys)
+                seqs, q0 = seqs[order], q0[order]
+                plan.count = int(seqs.size)
+                tag = f"talking:{h}:{hkv}:{d}:{s.window or 0}:{s.chunk or 0}"
+                plan.seq_name, plan.q0_name = f"attention_seq:{tag}", f"attention_q0:{tag}"
+                shape.add(plan.seq_name, seqs)
+                shape.add(plan.q0_name, q0)
+            shape.launch_key.append((key, "talking_mfma", shape.num_decode, plan.count))
+            return
         if self.talking:
             # a token's heads stay together in one workgroup; single tokens with many keys share
             # them among workgroups (bfloat16 only: float32 keeps one order of summation whatever
@@ -353,6 +371,16 @@ class PagedAttention(Mixer):
             raise RuntimeError(f"{self.name}: the step was not prepared for this mixer "
                                "(the step function calls prepare() on every part)")
         q = qkv[:, : h * d]
+        if plan.kernel == "talking_mfma":
+            floats = ops.attention_talking_mfma_scratch_floats(q.shape[0], h, hkv, self.value_dim)
+            scratch = ctx.buffer("attn_talking_sums", (floats,), torch.float32)
+            ops.attention_talking_mfma(q, out, ctx.num_decode, h, hkv, d, self.value_dim, ctx.positions, ctx.token_seq,
+                                       ctx.cu_q, ctx.extras[plan.seq_name] if plan.count else None,
+                                       ctx.extras[plan.q0_name] if plan.count else None, plan.count, tables,
+                                       cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale, scratch,
+                                       chunk=s.chunk, r1=self.r1, r2=self.r2, talk=self.talk,
+                                       sink=getattr(s, "fixed_sink", None))
+            return
         if self.talking:
             floats = ops.attention_talking_scratch_floats(q.shape[0], h, self.value_dim, plan.nsplit)
             scratch = ctx.buffer("attn_talking_scratch", (floats,), torch.float32)

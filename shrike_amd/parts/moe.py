@@ -14,7 +14,9 @@ class MixtureOfExperts(FeedForward):
     matrices are stacked [experts, ...] when the weights are loaded and every (token, chosen
     expert) pair is multiplied by its own expert's rows on the device, chosen there: nothing of
     the routing is read on the host, so steps are recorded into graphs.  The shared expert is
-    the framework's dense gated product; its output is the sum's first term."""
+    the framework's dense gated product; its output is the sum's first term.  From a few
+    tokens on, bfloat16 steps list each expert's pairs on the device and run the two products
+    per expert on the matrix units, so that an expert's matrices are read once a step."""
 
     launches_follow_shape = True
 
@@ -79,8 +81,12 @@ class MixtureOfExperts(FeedForward):
             self.linear(act, self.shared[1], shared_out)
         act_buf = ctx.buffer("moe_act", (n * s.top, s.expert_size), ctx.dtype)
         out = ctx.buffer("moe_out", (n, self.width), ctx.dtype)
+        scratch = None
+        if ops.moe_grouped(n, self.width, s.expert_size, ctx.dtype):
+            scratch = ctx.buffer("moe_scratch", (ops.moe_grouped_scratch_bytes(n, self.width, s.experts, s.top),),
+                                 torch.uint8)
         ops.moe_experts(x, chosen, weights, self.w_gate, self.w_up, self.w_down, act_buf, out, s.activation,
-                        add=shared_out)
+                        add=shared_out, scratch=scratch)
         return out
 
 

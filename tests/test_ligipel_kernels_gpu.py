@@ -182,7 +182,7 @@ def test_mixed_head_attention_against_the_plain_form(ops, dtype, H, G, D, V, n, 
     whole = run_talking(ops, q, k, v, r1, r2, talk, window, scale, dtype, page_size, [n])
     close(whole, want.reshape(n, H * V), dtype, "whole")
     # portions down to two tokens, then single tokens: the same bits in float32
-    cuts = [5, 2, 17, 2, 3] + [1] * (n - 29)
+    cuts = [5, 2, 17, 2, 3] + [1] * (n - 29) if n > 29 else [3, 2] + [1] * (n - 5)
     pieces = run_talking(ops, q, k, v, r1, r2, talk, window, scale, dtype, page_size, cuts)
     close(pieces, want.reshape(n, H * V), dtype, "pieces")
     if dtype == torch.float32:
@@ -386,14 +386,16 @@ def test_rotation_of_float32_rows(ops, heads, dim, rot, base):
     torch.manual_seed(dim)
     n, off, ld = 9, 5, 5 + heads * dim + 3
     x = torch.randn(n, ld)
-    positions = torch.tensor([0, 1, 2, 77, 1000, 4095, 30000, 3, 64])
+    positions = torch.tensor([0, 1, 2, 77, 64, 4095, 30000, 3, 1000])
     inv = torch.tensor([base ** (-2.0 * i / rot) for i in range(rot // 2)], dtype=torch.float32) if rot else None
     got = dev(x)
     ops.rotate_half_rows(got, off, heads, dim, rot, None if inv is None else dev(inv), i32(positions), 0.37)
     want = x.double().clone()
     want[:, off:off + heads * dim] = (plain.rotate_half(x[:, off:off + heads * dim].double().view(n, heads, dim),
                                                         positions, rot, base) * 0.37).reshape(n, heads * dim)
-    close(got, want, torch.float32, tol=2e-5)
+    # angles are 32-bit products of a position and a frequency: at position p they are p * 2^-24 off at most
+    close(got[:5], want[:5], torch.float32, tol=2e-5)
+    close(got, want, torch.float32, tol=30000 * 2.0**-23)
     assert torch.equal(got[:, :off].cpu(), x[:, :off]) and torch.equal(got[:, off + heads * dim:].cpu(), x[:, off + heads * dim:])
 
 
@@ -513,3 +515,140 @@ def test_experts_products_against_the_plain_form(ops, dtype, n, width, ff, exper
         assert torch.equal(alone[0], out[t])
     else:
         close(alone[0], out[t], dtype)
+
+
+# ------------------------------------------------------------------ the same on the matrix units (bfloat16)
+
+def run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, scale, page_size, sink=0.0):
+    """seqs: {name: (q, k, v)}; steps: lists of (name, start, count), single tokens first.  Every
+    sequence's keys and values are in the cache beforehand."""
+    dtype = torch.bfloat16
+    names = list(seqs)
+    pages = sum(-(-seqs[s][0].shape[0] // page_size) for s in names) + 5
+    perm = torch.randperm(pages, generator=torch.Generator().manual_seed(pages)).tolist()
+    slab = ops.key_slab(D)
+    k_pool = torch.full(ops.key_pool_shape(pages, G, page_size, D), float("nan"))  # what no one wrote is not a number
+    v_pool = torch.full((pages, G, V, page_size), float("nan"))
+    table_of, width = {}, max(-(-seqs[s][0].shape[0] // page_size) for s in names)
+    for s in names:
+        q, k, v = seqs[s]
+        table = [perm.pop() for _ in range(-(-q.shape[0] // page_size))]
+        for j in range(q.shape[0]):
+            k_pool[table[j // page_size], :, :, j % page_size, :] = k[j].view(G, D // slab, slab)
+            v_pool[table[j // page_size], :, :, j % page_size] = v[j]
+        table_of[s] = table + [-1] * (width - len(table))
+    k_pool, v_pool = dev(k_pool, dtype), dev(v_pool, dtype)
+    got = {s: torch.zeros(seqs[s][0].shape[0], H * V, dtype=dtype, device="cuda") for s in names}
+    for step in steps:
+        starts, lens = [st for _, st, _ in step], [c for _, _, c in step]
+        positions, token_seq, cu = step_arrays(starts, lens)
+        single = sum(1 for c in lens if c == 1)
+        assert all(c == 1 for c in lens[:single]) and all(c > 1 for c in lens[single:])
+        tile_seq, tile_q0 = [], []
+        for idx in range(single, len(step)):
+            for q0 in range(0, lens[idx], 16):
+                tile_seq.append(idx)
+                tile_q0.append(q0)
+        rows = dev(torch.cat([seqs[s][0][st:st + c].reshape(c, H * D) for s, st, c in step]), dtype)
+        n = rows.shape[0]
+        out = torch.empty(n, H * V, dtype=dtype, device="cuda")
+        scratch = torch.empty(ops.attention_talking_mfma_scratch_floats(n, H, G, V), device="cuda")
+        ops.attention_talking_mfma(rows, out, single, H, G, D, V, positions, token_seq, cu,
+                                   i32(tile_seq) if tile_seq else None, i32(tile_q0) if tile_q0 else None, len(tile_seq),
+                                   i32([table_of[s] for s, _, _ in step]), k_pool, v_pool, page_size, window, scale, scratch,
+                                   r1=None if r1 is None else dev(r1), r2=None if r2 is None else dev(r2),
+                                   talk=None if talk is None else dev(talk), sink=sink)
+        at = 0
+        for s, st, c in step:
+            got[s][st:st + c] = out[at:at + c]
+            at += c
+    return got
+
+
+@pytest.mark.parametrize("H, G, D, V, window, page_size", [
+    (4, 2, 32, 16, 7, 16),       # a window smaller than a page; values smaller than keys
+    (3, 1, 24, 40, 33, 8),       # a head size that is no multiple of 32, value blocks with a ragged end
+    (2, 2, 64, 64, None, 16),    # no window
+    (6, 3, 16, 8, 64, 8),
+    (8, 8, 128, 128, 100, 16),   # as many key/value heads as heads: value heads in several passes
+    (20, 1, 8, 24, 50, 32),      # more heads of a key/value head than a tile has rows
+    (4, 2, 256, 256, 45, 16),
+])
+def test_mixed_head_attention_on_the_matrix_units(ops, H, G, D, V, window, page_size):
+    dtype = torch.bfloat16
+    assert ops.attention_talking_supports_mfma(D, V, page_size, H * D)
+    lens = {"a": 150, "b": 37, "c": 1, "d": 70}
+    seqs, want = {}, {}
+    _, _, _, r1, r2, talk = talking_case(H, G, D, V, 1, 77, window)
+    talk = talk.to(dtype).float()  # (the weight file holds bfloat16)
+    for idx, (s, n) in enumerate(lens.items()):
+        q, k, v, _, _, _ = talking_case(H, G, D, V, n, 300 + idx, window)
+        seqs[s] = tuple(t.to(dtype).float() for t in (q, k, v))
+        qd, kd, vd = (t.double() for t in seqs[s])
+        want[s] = plain.mixed_head_attention(qd, kd, vd, 0.3, window, r1.double(), r2.double(), talk.double())
+    steps = [
+        [("c", 0, 1), ("a", 0, 40), ("b", 0, 2)],               # a first token alone, a portion, a two-token portion
+        [("a", 40, 1), ("b", 2, 1)],                            # single tokens only
+        [("b", 3, 1), ("a", 41, 17), ("d", 0, 33)],             # mixed; tiles with ragged ends
+        [("a", 58, 1), ("d", 33, 1), ("b", 4, 33)],
+        [("d", 34, 36), ("a", 59, 91)],                         # portions only, far into their sequences
+    ]
+    got = run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, 0.3, page_size)
+    for s, n in lens.items():
+        close(got[s], want[s].reshape(n, H * V), dtype, f"sequence {s}", tol=2e-2)
+
+
+@pytest.mark.parametrize("cuts", ["whole", "decode"])
+def test_the_window_ends_where_it_should_on_the_matrix_units(ops, cuts):
+    H, G, D, V, page_size, n = 2, 1, 16, 16, 16, 300
+    for target, window in [(15, 16), (16, 33), (63, 64), (64, 65), (3, 290), (130, 136), (200, 1), (31, 32), (32, 1)]:
+        g = torch.Generator().manual_seed(target)
+        q = torch.randn(n, H, D, generator=g) * 0.1
+        k = torch.randn(n, G, D, generator=g) * 0.1
+        v = torch.randn(n, G, V, generator=g) * 0.01
+        q[:, :, 0] = 6.0
+        k[target, 0, 0] = 6.0
+        v[target, 0, 0] = 100.0
+        r1, r2 = torch.tensor([0.5, 0.0]), torch.tensor([1.0, 3.0])
+        talk = torch.tensor([[1.0, 0.0], [0.25, 0.75]])
+        steps = [[("s", 0, n)]] if cuts == "whole" else [[("s", 0, target + 1)]] + [[("s", t, 1)] for t in range(target + 1, n)]
+        got = run_talking_mfma(ops, {"s": (q, k, v)}, steps, H, G, D, V, r1, r2, talk, window, 1.0, page_size)["s"].float().cpu()
+        seen = got[:, 0].abs() > 30.0
+        want = torch.zeros(n, dtype=torch.bool)
+        want[target:min(n, target + window)] = True
+        assert torch.equal(seen, want), f"target {target} window {window}: seen at {seen.nonzero().flatten().tolist()[:8]}.."
+
+
+@pytest.mark.parametrize("n, width, ff, experts, top, shared", [(4, 64, 24, 5, 2, True), (7, 104, 32, 4, 4, False),
+                                                                (40, 128, 64, 8, 1, True), (130, 72, 40, 9, 3, False),
+                                                                (300, 256, 96, 6, 2, True), (33, 64, 8, 70, 6, False)])
+def test_experts_products_per_expert_on_the_matrix_units(ops, n, width, ff, experts, top, shared):
+    dtype = torch.bfloat16
+    assert ops.moe_grouped(n, width, ff, dtype)
+    torch.manual_seed(n + width)
+    x = torch.randn(n, width).to(dtype)
+    wg, wu = (torch.randn(experts, ff, width) * width**-0.5).to(dtype), (torch.randn(experts, ff, width) * width**-0.5).to(dtype)
+    wd = (torch.randn(experts, width, ff) * ff**-0.5).to(dtype)
+    chosen = torch.stack([torch.randperm(experts)[:top] for _ in range(n)]).to(torch.int32)
+    chosen[: n // 3] = torch.arange(top, dtype=torch.int32)  # many tokens on the same experts: lists longer than a tile
+    weights = torch.rand(n, top)
+    weights = weights / weights.sum(dim=-1, keepdim=True)
+    add = torch.randn(n, width).to(dtype) if shared else None
+    outs = []
+    for grouped in (False, True):
+        act = torch.full((n * top, ff), float("nan"), dtype=dtype, device="cuda")
+        out = torch.empty(n, width, dtype=dtype, device="cuda")
+        scratch = torch.empty(ops.moe_grouped_scratch_bytes(n, width, experts, top), dtype=torch.uint8, device="cuda") \
+            if grouped else None
+        ops.moe_experts(dev(x), dev(chosen), dev(weights), dev(wg), dev(wu), dev(wd), act, out, "silu",
+                        add=None if add is None else dev(add), scratch=scratch)
+        outs.append(out.float().cpu())
+    want = torch.zeros(n, width, dtype=torch.float64) if add is None else add.double().clone()
+    xd = x.double()
+    for t in range(n):
+        for j in range(top):
+            e = int(chosen[t, j])
+            hidden = (plain.silu(wg[e].double() @ xd[t]) * (wu[e].double() @ xd[t])).to(dtype).double()
+            want[t] += weights[t, j].double() * (wd[e].double() @ hidden)
+    close(outs[1], want, dtype, "per expert", tol=2e-2)
+    close(outs[1], outs[0], dtype, "against the pair-by-pair kernel", tol=2e-2)
