@@ -326,7 +326,7 @@ def kernel_breakdown(engine, steps: int = 3, before_step=None) -> dict:
              "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample",
              "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows", "embed_pairs", "qkv_store",
              "latent_prepare", "rotate_heads", "latent_attention", "latent_attention_mfma", "gemm_batched", "mlstm_scan", "headnorm_gate",
-             "xielu", "layernorm", "add_layernorm", "attention_talking", "conv_silu", "dt_softplus", "selective_scan",
+             "xielu", "layernorm", "add_layernorm", "attention_talking", "attention_talking_mfma", "conv_silu", "dt_softplus", "selective_scan",
              "rotate_half_rows", "retention_scan", "moe_route", "moe_experts", "mix_history", "scale_softcap"]
     names = [n for n in names if hasattr(ops, n)]
     spans: list[tuple[str, object, object]] = []

@@ -318,22 +318,23 @@ int shk_attention_talking(const void* q, int q_stride, void* out, int dtype, int
 // running maximum and sum), and the sums are mixed: o_h = sum_g talk[h, g] U[g, c(h)].  The step's
 // first num_single tokens are single tokens of sequences 0 .. num_single - 1; prompt portions come
 // as num_tiles tiles of 16 queries (tile_seq, tile_q0 counted from the portion's first query; cu_q[s]
-// = sequence s's first row).  scratch: shk_attention_talking_mfma_scratch_floats(...) floats.
+// = sequence s's first row).  nsplit > 1 shares every single token's keys among that many workgroups,
+// whose sums are joined in order.  scratch: shk_attention_talking_mfma_scratch_floats(...) floats.
 int shk_attention_talking_supports_mfma(int head_dim, int v_dim, int page_size, int q_stride);
-long long shk_attention_talking_mfma_scratch_floats(int n, int heads, int kv_heads, int v_dim);
+long long shk_attention_talking_mfma_scratch_floats(int n, int num_single, int heads, int kv_heads, int v_dim, int nsplit);
 int shk_attention_talking_bf16(const void* q, int q_stride, void* out, int n, int num_single, int num_tiles,
                                int heads, int kv_heads, int head_dim, int v_dim, const int32_t* positions,
                                const int32_t* token_seq, const int32_t* cu_q, const int32_t* tile_seq,
                                const int32_t* tile_q0, const int32_t* tables, int table_stride, const void* k_pool,
                                const void* v_pool, int page_size, int num_pages, int window, int chunk, float scale,
                                const float* r1, const float* r2, const float* talk, int has_sink, float sink,
-                               float* scratch, void* stream);
+                               float* scratch, int nsplit, void* stream);
 
 // The selective scan of Mamba and its causal convolution (ssm.hip).  A request's slot holds S
 // [inner, states] float32 and then the convolution's last taps - 1 inputs [(taps - 1), inner].
 // shk_conv_silu: y[t, c] = silu(bias[c] + sum_k taps[c, num_taps - 1 - k] * x[t - k, c]) over the
 // sequence's earlier inputs (rows of this step, else the slot's kept ones, zero before position 0).
-// shk_dt_softplus: dt[t, c] = softplus(b[c] + sum_r w[c, r] * low[t, r]), float32.
+// shk_dt_softplus: dt[t, c] = softplus(b[c] + sum_r w[r, c] * low[t, r]), float32; w [rank, inner].
 // shk_selective_scan: S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n, y_c = sum_n S[c, n] C_n +
 // dskip_c x_c, out = y * silu(z); A = -exp(a_log); B and C are columns b_off, c_off of bc (float32);
 // `raw` are the convolution's inputs of the step, of which the slot keeps the last taps - 1.

@@ -255,7 +255,7 @@ __global__ void __launch_bounds__(256)
                         int window, int chunk, float scale_l2, const float* __restrict__ r1,
                         const float* __restrict__ r2, int has_sink, float sink_l2, const int32_t* __restrict__ cu_q,
                         const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int tiles_mode,
-                        int first_token, int vh_pass) {
+                        int nsplit, float* __restrict__ partial, int vh_pass) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int i = lane % 16, kg = lane / 16;
   const int group = heads / kv_heads;
@@ -276,7 +276,7 @@ __global__ void __launch_bounds__(256)
   } else {
     const int subs = (group + 15) / 16;
     if (unit >= kv_heads * subs) return;
-    t = first_token + blockIdx.x;
+    t = blockIdx.x / nsplit;
     seq = token_seq[t];
     ck = unit / subs;
     const int within = (unit % subs) * 16 + i;
@@ -307,12 +307,18 @@ __global__ void __launch_bounds__(256)
   tf32x4 o[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) o[b] = tf32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = has_sink ? sink_l2 : -INFINITY;
-  float l_run = has_sink ? 1.f : 0.f;
+  // single tokens with many keys: share `share` of nsplit takes a run of the chunks (the sink is the first one's)
+  const int share = tiles_mode ? 0 : blockIdx.x % nsplit;
+  const int chunk_lo = lo_min / 32, chunk_hi = pos_max / 32;
+  const int per_share = (chunk_hi - chunk_lo + nsplit) / nsplit;
+  const int j_begin = (chunk_lo + share * per_share) * 32;
+  const int j_end = min(pos_max, (chunk_lo + (share + 1) * per_share) * 32 - 1);
+  float m_run = has_sink && share == 0 ? sink_l2 : -INFINITY;
+  float l_run = has_sink && share == 0 ? 1.f : 0.f;
   const int slab = key_slab(head_dim);
   const size_t k_head = static_cast<size_t>(page_size) * head_dim;  // elements of a page's head
   const size_t v_head = static_cast<size_t>(page_size) * v_dim;
-  for (int j0 = lo_min / 32 * 32; j0 <= pos_max; j0 += 32) {
+  for (int j0 = j_begin; j0 <= j_end; j0 += 32) {
     // scores: A row m of product t2 is the key j0 + 8 (m / 4) + 4 t2 + m % 4
     tf32x4 s[2];
 #pragma unroll
@@ -405,8 +411,17 @@ __global__ void __launch_bounds__(256)
   }
   if (!valid) return;
   // this lane holds value elements (b % vb) * 16 + 4 kg + r of its row
-  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  float inv = l_run > 0.f ? 1.f / l_run : 0.f;
   float* dst = u_out + (static_cast<size_t>(t) * heads + head) * kv_heads * v_dim;
+  if (nsplit > 1) {  // the share's sums as they stand, then its maximum and denominator
+    const int gv = kv_heads * v_dim;
+    dst = partial + ((static_cast<size_t>(t) * heads + head) * nsplit + share) * (gv + 2);
+    inv = 1.f;
+    if (kg == 0 && blockIdx.z == 0) {
+      dst[gv] = m_run;
+      dst[gv + 1] = l_run;
+    }
+  }
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
     const int cvl = b / vb;
@@ -417,6 +432,28 @@ __global__ void __launch_bounds__(256)
       if (d < v_dim) dst[static_cast<size_t>(cv0 + cvl) * v_dim + d] = o[b][r] * inv;
     }
   }
+}
+
+// u[t, g, :] of single tokens from their shares: sum_z o_z 2^(m_z - m) / sum_z l_z 2^(m_z - m)
+__global__ void __launch_bounds__(256)
+    talking_join_kernel(const float* __restrict__ partial, float* __restrict__ u_out, int heads, int gv, int nsplit) {
+  const int t = blockIdx.y;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= heads * gv) return;
+  const int head = idx / gv, rest = idx % gv;
+  const float* base = partial + (static_cast<size_t>(t) * heads + head) * nsplit * (gv + 2);
+  float m = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) m = fmaxf(m, base[static_cast<size_t>(z) * (gv + 2) + gv]);
+  float den = 0.f, val = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = base[static_cast<size_t>(z) * (gv + 2) + gv];
+    if (mz > -INFINITY) {
+      const float w = __builtin_amdgcn_exp2f(mz - m);
+      den = fmaf(base[static_cast<size_t>(z) * (gv + 2) + gv + 1], w, den);
+      val = fmaf(base[static_cast<size_t>(z) * (gv + 2) + rest], w, val);
+    }
+  }
+  u_out[(static_cast<size_t>(t) * heads + head) * gv + rest] = den > 0.f ? val / den : 0.f;
 }
 
 // out[t, h, d] = sum_g talk[h, g] * U[t, g, c(h), d]   (talk null: U[t, h, c(h), d])
@@ -508,8 +545,10 @@ extern "C" int shk_attention_talking_supports_mfma(int head_dim, int v_dim, int 
   return head_dim % 8 == 0 && head_dim <= 256 && v_dim >= 1 && v_dim <= 256 && page_size % 8 == 0 && q_stride % 8 == 0;
 }
 
-extern "C" long long shk_attention_talking_mfma_scratch_floats(int n, int heads, int kv_heads, int v_dim) {
-  return static_cast<long long>(n) * heads * kv_heads * v_dim;
+extern "C" long long shk_attention_talking_mfma_scratch_floats(int n, int num_single, int heads, int kv_heads, int v_dim,
+                                                               int nsplit) {
+  const long long gv = static_cast<long long>(kv_heads) * v_dim;
+  return static_cast<long long>(n) * heads * gv + (nsplit > 1 ? static_cast<long long>(num_single) * heads * nsplit * (gv + 2) : 0);
 }
 
 namespace shk {
@@ -520,12 +559,12 @@ static void launch_talking_mfma(dim3 grid, hipStream_t s, const bf16* q, int q_s
                                 const int32_t* tables, int table_stride, const bf16* k_pool, const bf16* v_pool,
                                 int page_size, int num_pages, int window, int chunk, float scale_l2, const float* r1,
                                 const float* r2, int has_sink, float sink_l2, const int32_t* cu_q,
-                                const int32_t* tile_seq, const int32_t* tile_q0, int tiles_mode, int first_token,
-                                int vh_pass) {
+                                const int32_t* tile_seq, const int32_t* tile_q0, int tiles_mode, int nsplit,
+                                float* partial, int vh_pass) {
   talking_mfma_kernel<KS, NB><<<grid, 256, 0, s>>>(q, q_stride, u, heads, kv_heads, head_dim, v_dim, positions, token_seq,
                                                    tables, table_stride, k_pool, v_pool, page_size, num_pages, window,
                                                    chunk, scale_l2, r1, r2, has_sink, sink_l2, cu_q, tile_seq, tile_q0,
-                                                   tiles_mode, first_token, vh_pass);
+                                                   tiles_mode, nsplit, partial, vh_pass);
 }
 
 }  // namespace shk
@@ -536,7 +575,8 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
                                           const int32_t* tile_q0, const int32_t* tables, int table_stride,
                                           const void* k_pool, const void* v_pool, int page_size, int num_pages,
                                           int window, int chunk, float scale, const float* r1, const float* r2,
-                                          const float* talk, int has_sink, float sink, float* scratch, void* stream) {
+                                          const float* talk, int has_sink, float sink, float* scratch, int nsplit,
+                                          void* stream) {
   SHK_REQUIRE(n >= 0 && num_single >= 0 && num_single <= n && num_tiles >= 0 && heads > 0 && kv_heads > 0 &&
                   heads % kv_heads == 0,
               "attention_talking_bf16: bad sizes n=%d single=%d tiles=%d heads=%d kv_heads=%d", n, num_single, num_tiles,
@@ -557,6 +597,8 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
                   reinterpret_cast<uintptr_t>(v_pool) % 16 == 0,
               "attention_talking_bf16: operands must be 16-byte aligned");
   SHK_REQUIRE(n <= 65535 && num_tiles <= 0x7fffffff / 4, "attention_talking_bf16: at most 65535 tokens a call, got %d", n);
+  SHK_REQUIRE(nsplit >= 1 && nsplit <= 64, "attention_talking_bf16: 1 to 64 shares of a single token's keys, got %d", nsplit);
+  float* partial = scratch + static_cast<size_t>(n) * heads * kv_heads * v_dim;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float log2e = 1.4426950408889634f;
   const int ks = (head_dim + 31) / 32, vb = (v_dim + 15) / 16;
@@ -565,13 +607,12 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
   launch_talking_mfma<KS, NB>(grid, s, static_cast<const bf16*>(q), q_stride, scratch, heads, kv_heads, head_dim, v_dim, \
                               positions, token_seq, tables, table_stride, static_cast<const bf16*>(k_pool),             \
                               static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale * log2e, r1,  \
-                              r2, has_sink, sink * log2e, cu_q, tile_seq, tile_q0, mode, 0, vh_pass)
+                              r2, has_sink, sink * log2e, cu_q, tile_seq, tile_q0, mode, shares, partial, vh_pass)
 #define SHK_NB(KS)                                                                                                     \
   if (nb <= 2) SHK_GO(KS, 2);                                                                                          \
   else if (nb <= 4) SHK_GO(KS, 4);                                                                                     \
   else if (nb <= 8) SHK_GO(KS, 8);                                                                                     \
-  else if (nb <= 16) SHK_GO(KS, 16);                                                                                   \
-  else SHK_GO(KS, 32)
+  else SHK_GO(KS, 16)
 #define SHK_KS()                                                                                                       \
   if (ks <= 1) { SHK_NB(1); }                                                                                          \
   else if (ks <= 2) { SHK_NB(2); }                                                                                     \
@@ -579,14 +620,20 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
   else { SHK_NB(8); }
   if (num_single > 0) {
     // single tokens: a key/value head's query heads are a tile's rows; one value head a workgroup
-    const int mode = 0, vh_pass = 1, nb = vb;
+    const int mode = 0, vh_pass = 1, nb = vb, shares = nsplit;
     const int units = kv_heads * ((group + 15) / 16);
-    dim3 grid(num_single, (units + 3) / 4, kv_heads);
+    dim3 grid(num_single * nsplit, (units + 3) / 4, kv_heads);
     SHK_KS()
+    if (nsplit > 1) {
+      const int items = heads * kv_heads * v_dim;
+      talking_join_kernel<<<dim3((items + 255) / 256, num_single), 256, 0, s>>>(partial, scratch, heads, kv_heads * v_dim,
+                                                                              nsplit);
+    }
   }
   if (num_tiles > 0) {
-    const int mode = 1;
-    const int vh_pass = max(1, min(kv_heads, 32 / vb));
+    // (8 blocks of sums a pass where a head's values allow it: two wavefronts then share a SIMD's registers)
+    const int mode = 1, shares = 1;
+    const int vh_pass = max(1, min(kv_heads, 8 / vb));
     const int nb = vh_pass * vb;
     dim3 grid(num_tiles, (heads + 3) / 4, (kv_heads + vh_pass - 1) / vh_pass);
     SHK_KS()

@@ -59,23 +59,38 @@ __global__ void __launch_bounds__(256)
   y[static_cast<size_t>(t) * inner + c] = from_float<T>(silu_f(acc));
 }
 
-// dt[t, c] = softplus(b[c] + sum_r W[c, r] * low[t, r]) in float32
+constexpr int kDtTokens = 8;  // tokens a workgroup: the matrix is read once for all of them
+
+// dt[t, c] = softplus(b[c] + sum_r W[r, c] * low[t, r]) in float32; W is given transposed, [rank, inner], so
+// that neighbouring channels' weights are neighbours in memory.  A token's sum runs over r in ascending
+// order whatever else is in the step.
 __global__ void __launch_bounds__(256)
-    dt_softplus_kernel(const float* __restrict__ low, int ld, const float* __restrict__ w, const float* __restrict__ b,
-                       int rank, int inner, float* __restrict__ dt) {
-  extern __shared__ float lows[];
-  const int t = blockIdx.y;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) lows[r] = low[static_cast<size_t>(t) * ld + r];
+    dt_softplus_kernel(const float* __restrict__ low, int ld, const float* __restrict__ wt, const float* __restrict__ b,
+                       int rank, int inner, float* __restrict__ dt, int n) {
+  extern __shared__ float lows[];  // [kDtTokens, rank]
+  const int t0 = blockIdx.y * kDtTokens;
+  const int count = min(kDtTokens, n - t0);
+  for (int i = threadIdx.x; i < count * rank; i += blockDim.x)
+    lows[i] = low[static_cast<size_t>(t0 + i / rank) * ld + i % rank];
   __syncthreads();
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= inner) return;
-  float acc = b[c];
-  const float* wr = w + static_cast<size_t>(c) * rank;
-  for (int r = 0; r < rank; ++r) acc = fmaf(wr[r], lows[r], acc);
-  dt[static_cast<size_t>(t) * inner + c] = softplus_f(acc);
+  float acc[kDtTokens];
+#pragma unroll
+  for (int k = 0; k < kDtTokens; ++k) acc[k] = b[c];
+  for (int r = 0; r < rank; ++r) {
+    const float w = wt[static_cast<size_t>(r) * inner + c];
+#pragma unroll
+    for (int k = 0; k < kDtTokens; ++k)
+      if (k < count) acc[k] = fmaf(w, lows[k * rank + r], acc[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < kDtTokens; ++k)
+    if (k < count) dt[static_cast<size_t>(t0 + k) * inner + c] = softplus_f(acc[k]);
 }
 
 constexpr int kStatesPerLane = 8;
+constexpr int kScanBlock = 16;  // tokens whose inputs are fetched together
 
 // One sequence's tokens for a block of channels.  LANES lanes share a channel's states
 // (LANES * 8 >= states); a wavefront holds 64 / LANES channels.
@@ -87,11 +102,15 @@ __global__ void __launch_bounds__(256)
                           int K, const T* __restrict__ raw, int ld_raw, const int32_t* __restrict__ positions,
                           const int32_t* __restrict__ cu_q, const int32_t* __restrict__ slots,
                           float* __restrict__ state, long long slot_stride, T* __restrict__ out) {
+  // Tokens go by in blocks of kScanBlock: a block's B and C (the same for every channel) are staged in
+  // LDS by the workgroup, and a lane fetches its channel's step sizes, inputs and gates of the block at
+  // once, so that the walk over the tokens waits for memory once a block and not once a token.
+  extern __shared__ float bcs[];  // [kScanBlock][2 * states]
   const int seq = blockIdx.y;
   const int unit = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;  // channel
   const int part = threadIdx.x % LANES;
-  if (unit >= inner) return;
-  const int c = unit;
+  const bool active = unit < inner;
+  const int c = active ? unit : inner - 1;
   const int first = cu_q[seq], last = cu_q[seq + 1];
   if (last <= first) return;
   float* slot = state + static_cast<size_t>(slots[seq]) * slot_stride;
@@ -105,29 +124,47 @@ __global__ void __launch_bounds__(256)
     A[i] = n < states ? -expf(a_log[static_cast<size_t>(c) * states + n]) : 0.f;
   }
   const float dc = dskip[c];
-  for (int t = first; t < last; ++t) {
-    const float step = dt[static_cast<size_t>(t) * inner + c];
-    const float xv = to_float(x[static_cast<size_t>(t) * inner + c]);
-    const float* bt = bc + static_cast<size_t>(t) * ld_bc + b_off;
-    const float* ct = bc + static_cast<size_t>(t) * ld_bc + c_off;
-    const float dx = step * xv;
-    float y = 0.f;
+  for (int t0 = first; t0 < last; t0 += kScanBlock) {
+    const int count = min(kScanBlock, last - t0);
+    __syncthreads();  // (the block before has been read)
+    for (int i = threadIdx.x; i < count * 2 * states; i += 256) {
+      const int tt = i / (2 * states), j = i % (2 * states);
+      bcs[i] = bc[static_cast<size_t>(t0 + tt) * ld_bc + (j < states ? b_off + j : c_off + j - states)];
+    }
+    float stepv[kScanBlock], xs[kScanBlock], gs[kScanBlock];
 #pragma unroll
-    for (int i = 0; i < kStatesPerLane; ++i) {
-      const int n = part * kStatesPerLane + i;
-      if (n < states) {
-        S[i] = fmaf(expf(step * A[i]), S[i], dx * bt[n]);
-        y = fmaf(S[i], ct[n], y);
+    for (int k = 0; k < kScanBlock; ++k) {
+      const int t = t0 + (k < count ? k : 0);
+      stepv[k] = dt[static_cast<size_t>(t) * inner + c];
+      xs[k] = to_float(x[static_cast<size_t>(t) * inner + c]);
+      gs[k] = to_float(z[static_cast<size_t>(t) * ldz + c]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kScanBlock; ++k) {
+      if (k >= count) break;
+      const float step = stepv[k], xv = xs[k];
+      const float* bt = bcs + k * 2 * states;
+      const float* ct = bt + states;
+      const float dx = step * xv;
+      float y = 0.f;
+#pragma unroll
+      for (int i = 0; i < kStatesPerLane; ++i) {
+        const int n = part * kStatesPerLane + i;
+        if (n < states) {
+          S[i] = fmaf(expf(step * A[i]), S[i], dx * bt[n]);
+          y = fmaf(S[i], ct[n], y);
+        }
+      }
+#pragma unroll
+      for (int off = LANES / 2; off > 0; off >>= 1) y += __shfl_xor(y, off, kWave);
+      if (part == 0 && active) {
+        y = fmaf(dc, xv, y);
+        out[static_cast<size_t>(t0 + k) * inner + c] = from_float<T>(y * silu_f(gs[k]));
       }
     }
-#pragma unroll
-    for (int off = LANES / 2; off > 0; off >>= 1) y += __shfl_xor(y, off, kWave);
-    if (part == 0) {
-      y = fmaf(dc, xv, y);
-      const float g = to_float(z[static_cast<size_t>(t) * ldz + c]);
-      out[static_cast<size_t>(t) * inner + c] = from_float<T>(y * silu_f(g));
-    }
   }
+  if (!active) return;
 #pragma unroll
   for (int i = 0; i < kStatesPerLane; ++i) {
     const int n = part * kStatesPerLane + i;
@@ -181,6 +218,14 @@ __global__ void __launch_bounds__(256)
 }
 
 constexpr int kRowsPerLane = 16;
+constexpr int kRetBlock = 8;  // tokens whose inputs are fetched together
+
+// the heads that the columns of one workgroup (256 / lanes of them) can belong to
+inline int retention_heads_a_workgroup(int lanes, int heads, int v_dim) {
+  const int per_wg = 256 / lanes;
+  const int most = (per_wg + v_dim - 2) / v_dim + 1;
+  return most < heads ? most : heads;
+}
 
 // One sequence's tokens for one (head, value column); LANES lanes share the column's rows
 // of S (LANES * 16 >= dim).
@@ -190,12 +235,22 @@ __global__ void __launch_bounds__(256)
                           const float* __restrict__ decay, int heads, int dim, int v_dim,
                           const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
                           const int32_t* __restrict__ slots, float* __restrict__ state, long long slot_stride,
-                          float* __restrict__ out) {
+                          float* __restrict__ out, int block) {
+  // Tokens go by in blocks of `block` (at most kRetBlock): the queries and keys of the heads that this workgroup's columns
+  // belong to are staged in LDS by the workgroup ([token][head][q | k]), a lane fetches its column's
+  // values of the block at once: the walk waits for memory once a block.
+  extern __shared__ float qks[];
   const int seq = blockIdx.y;
-  const int unit = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;  // (head, column)
+  const int per_wg = 256 / LANES;
+  const int unit_raw = blockIdx.x * per_wg + threadIdx.x / LANES;  // (head, column)
   const int part = threadIdx.x % LANES;
-  if (unit >= heads * v_dim) return;
+  const int units = heads * v_dim;
+  const bool active = unit_raw < units;
+  const int unit = active ? unit_raw : units - 1;
   const int h = unit / v_dim, col = unit % v_dim;
+  const int h_lo = blockIdx.x * per_wg / v_dim;
+  const int h_hi = min(units - 1, blockIdx.x * per_wg + per_wg - 1) / v_dim;
+  const int nh = h_hi - h_lo + 1;
   const int first = cu_q[seq], last = cu_q[seq + 1];
   if (last <= first) return;
   float* srow = state + static_cast<size_t>(slots[seq]) * slot_stride + static_cast<size_t>(unit) * dim;
@@ -207,24 +262,41 @@ __global__ void __launch_bounds__(256)
     S[i] = (d < dim && !fresh) ? srow[d] : 0.f;
   }
   const float a = decay[h];
-  for (int t = first; t < last; ++t) {
-    const float* row = proj + static_cast<size_t>(t) * ld;
-    const float* qt = row + q_off + h * dim;
-    const float* kt = row + k_off + h * dim;
-    const float vv = row[v_off + h * v_dim + col];
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < kRowsPerLane; ++i) {
-      const int d = part * kRowsPerLane + i;
-      if (d < dim) {
-        S[i] = fmaf(a, S[i], kt[d] * vv);
-        o = fmaf(S[i], qt[d], o);
-      }
+  for (int t0 = first; t0 < last; t0 += block) {
+    const int count = min(block, last - t0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < count * nh * 2 * dim; i += 256) {
+      const int tt = i / (nh * 2 * dim), rest = i % (nh * 2 * dim);
+      const int hh = rest / (2 * dim), j = rest % (2 * dim);
+      const float* row = proj + static_cast<size_t>(t0 + tt) * ld;
+      qks[i] = j < dim ? row[q_off + (h_lo + hh) * dim + j] : row[k_off + (h_lo + hh) * dim + j - dim];
     }
+    float vs[kRetBlock];
 #pragma unroll
-    for (int off = LANES / 2; off > 0; off >>= 1) o += __shfl_xor(o, off, kWave);
-    if (part == 0) out[static_cast<size_t>(t) * heads * v_dim + unit] = o;
+    for (int k = 0; k < kRetBlock; ++k)
+      vs[k] = proj[static_cast<size_t>(t0 + (k < count ? k : 0)) * ld + v_off + h * v_dim + col];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kRetBlock; ++k) {
+      if (k >= count) break;
+      const float* qt = qks + (static_cast<size_t>(k) * nh + (h - h_lo)) * 2 * dim;
+      const float* kt = qt + dim;
+      const float vv = vs[k];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < kRowsPerLane; ++i) {
+        const int d = part * kRowsPerLane + i;
+        if (d < dim) {
+          S[i] = fmaf(a, S[i], kt[d] * vv);
+          o = fmaf(S[i], qt[d], o);
+        }
+      }
+#pragma unroll
+      for (int off = LANES / 2; off > 0; off >>= 1) o += __shfl_xor(o, off, kWave);
+      if (part == 0 && active) out[static_cast<size_t>(t0 + k) * heads * v_dim + unit] = o;
+    }
   }
+  if (!active) return;
 #pragma unroll
   for (int i = 0; i < kRowsPerLane; ++i) {
     const int d = part * kRowsPerLane + i;
@@ -275,14 +347,13 @@ extern "C" int shk_conv_silu(const void* x, int ldx, const float* taps, const fl
 
 extern "C" int shk_dt_softplus(const float* low, int ld, const float* w, const float* b, int rank, int inner,
                                float* dt, int n, void* stream) {
-  SHK_REQUIRE(n >= 0 && inner > 0 && rank > 0 && rank <= 8192 && ld >= rank, "dt_softplus: bad sizes n=%d inner=%d rank=%d",
+  SHK_REQUIRE(n >= 0 && inner > 0 && rank > 0 && rank <= 1024 && ld >= rank, "dt_softplus: bad sizes n=%d inner=%d rank=%d",
               n, inner, rank);
   if (n == 0) return 0;
-  SHK_REQUIRE(n <= 65535, "dt_softplus: at most 65535 tokens a call, got %d", n);
   SHK_REQUIRE(low && w && b && dt, "dt_softplus: null pointer");
-  dim3 grid((inner + 255) / 256, n);
-  dt_softplus_kernel<<<grid, 256, rank * sizeof(float), static_cast<hipStream_t>(stream)>>>(low, ld, w, b, rank, inner,
-                                                                                           dt);
+  dim3 grid((inner + 255) / 256, (n + kDtTokens - 1) / kDtTokens);
+  dt_softplus_kernel<<<grid, 256, kDtTokens * rank * sizeof(float), static_cast<hipStream_t>(stream)>>>(
+      low, ld, w, b, rank, inner, dt, n);
   SHK_LAUNCH_CHECK("dt_softplus");
   return 0;
 }
@@ -307,7 +378,8 @@ extern "C" int shk_selective_scan(const float* dt, const void* x, const float* b
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int lanes = lanes_for(states, kStatesPerLane);
 #define SHK_GO(T, L)                                                                                                 \
-  selective_scan_kernel<T, L><<<dim3((inner + 256 / L - 1) / (256 / L), num_seqs), 256, 0, s>>>(                     \
+  selective_scan_kernel<T, L><<<dim3((inner + 256 / L - 1) / (256 / L), num_seqs), 256,                              \
+                                kScanBlock * 2 * states * sizeof(float), s>>>(                                       \
       dt, static_cast<const T*>(x), bc, ld_bc, b_off, c_off, static_cast<const T*>(z), ldz, a_log, dskip, inner,     \
       states, num_taps, static_cast<const T*>(raw), ld_raw, positions, cu_q, slots, state, slot_stride,              \
       static_cast<T*>(out))
@@ -367,9 +439,14 @@ extern "C" int shk_retention_scan(const float* proj, int ld, int q_off, int k_of
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int lanes = lanes_for(dim, kRowsPerLane);
   const int units = heads * v_dim;
+  const size_t a_token = static_cast<size_t>(retention_heads_a_workgroup(lanes, heads, v_dim)) * 2 * dim * sizeof(float);
+  SHK_REQUIRE(a_token <= 64000, "retention_scan: %d heads of %d elements a workgroup do not fit its LDS",
+              retention_heads_a_workgroup(lanes, heads, v_dim), dim);
+  const int block = static_cast<int>(64000 / a_token) < kRetBlock ? static_cast<int>(64000 / a_token) : kRetBlock;
+  const size_t lds = block * a_token;
 #define SHK_GO(L)                                                                                              \
-  retention_scan_kernel<L><<<dim3((units + 256 / L - 1) / (256 / L), num_seqs), 256, 0, s>>>(                  \
-      proj, ld, q_off, k_off, v_off, decay, heads, dim, v_dim, positions, cu_q, slots, state, slot_stride, out)
+  retention_scan_kernel<L><<<dim3((units + 256 / L - 1) / (256 / L), num_seqs), 256, lds, s>>>(                \
+      proj, ld, q_off, k_off, v_off, decay, heads, dim, v_dim, positions, cu_q, slots, state, slot_stride, out, block)
   switch (lanes) {
     case 1: SHK_GO(1); break;
     case 2: SHK_GO(2); break;

@@ -60,7 +60,7 @@ _SIGNATURES = {
     "shk_attention_talking": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _P, _P,
                               _P, _I, _F, _P, _I, _P],
     "shk_attention_talking_bf16": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I,
-                                   _I, _F, _P, _P, _P, _I, _F, _P, _P],
+                                   _I, _F, _P, _P, _P, _I, _F, _P, _I, _P],
     "shk_conv_silu": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, c_longlong, _I, _P, _I, _I, _P],
     "shk_dt_softplus": [_P, _I, _P, _P, _I, _I, _P, _I, _P],
     "shk_selective_scan": [_P, _P, _P, _I, _I, _I, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, c_longlong,
@@ -140,7 +140,7 @@ def load():
                                ("shk_selective_scan_state_floats", [_I, _I, _I]),
                                ("shk_retention_state_floats", [_I, _I, _I]),
                                ("shk_moe_grouped_scratch_bytes", [_I, _I, _I, _I]),
-                               ("shk_attention_talking_mfma_scratch_floats", [_I, _I, _I, _I])):
+                               ("shk_attention_talking_mfma_scratch_floats", [_I, _I, _I, _I, _I, _I])):
             fn = getattr(raw, name)
             fn.argtypes, fn.restype = argtypes, c_longlong
             setattr(lib, name, fn)

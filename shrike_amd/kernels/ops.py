@@ -781,16 +781,18 @@ def attention_talking_supports_mfma(head_dim: int, v_dim: int, page_size: int, q
     return bool(load().shk_attention_talking_supports_mfma(head_dim, v_dim, page_size, q_stride))
 
 
-def attention_talking_mfma_scratch_floats(n: int, heads: int, kv_heads: int, v_dim: int) -> int:
-    return int(load().shk_attention_talking_mfma_scratch_floats(n, heads, kv_heads, v_dim))
+def attention_talking_mfma_scratch_floats(n: int, heads: int, kv_heads: int, v_dim: int, num_single: int = 0,
+                                          nsplit: int = 1) -> int:
+    return int(load().shk_attention_talking_mfma_scratch_floats(n, num_single, heads, kv_heads, v_dim, nsplit))
 
 
 def attention_talking_mfma(q, out, num_single, heads, kv_heads, head_dim, v_dim, positions, token_seq, cu_q, tile_seq,
                            tile_q0, num_tiles, tables, k_pool, v_pool, page_size, window, scale, scratch, chunk=None,
-                           r1=None, r2=None, talk=None, sink=None) -> None:
+                           r1=None, r2=None, talk=None, sink=None, nsplit: int = 1) -> None:
     """attention_talking for bfloat16 on the matrix units.  The first num_single rows are single
     tokens of sequences 0 .. num_single - 1; the prompt portions after them are listed as
     num_tiles tiles of 16 queries (tile_seq, tile_q0: int32, q0 counted within the portion).
+    nsplit > 1 shares every single token's keys among that many workgroups.
     scratch: float32 of attention_talking_mfma_scratch_floats(...)."""
     _rows(q, "attention_talking_mfma q")
     n = q.shape[0]
@@ -800,7 +802,8 @@ def attention_talking_mfma(q, out, num_single, heads, kv_heads, head_dim, v_dim,
     for name, t, count in (("r1", r1, heads), ("r2", r2, heads), ("talk", talk, heads * heads)):
         if t is not None and (t.dtype != torch.float32 or t.numel() != count or not t.is_contiguous()):
             raise KernelError(f"attention_talking_mfma: {name} must be contiguous float32 of {count} values")
-    if scratch.dtype != torch.float32 or scratch.numel() < attention_talking_mfma_scratch_floats(n, heads, kv_heads, v_dim):
+    if scratch.dtype != torch.float32 or scratch.numel() < attention_talking_mfma_scratch_floats(
+            n, heads, kv_heads, v_dim, num_single, nsplit):
         raise KernelError("attention_talking_mfma: scratch is too small")
     if num_tiles and (tile_seq is None or tile_q0 is None or tile_seq.numel() < num_tiles or tile_q0.numel() < num_tiles):
         raise KernelError("attention_talking_mfma: the tile lists are shorter than num_tiles")
@@ -813,7 +816,7 @@ def attention_talking_mfma(q, out, num_single, heads, kv_heads, head_dim, v_dim,
         tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size, k_pool.shape[0], int(window or 0),
         int(chunk or 0), float(scale), None if r1 is None else _dev(r1, "r1"), None if r2 is None else _dev(r2, "r2"),
         None if talk is None else _dev(talk, "talk"), int(sink is not None), float(sink or 0.0),
-        _dev(scratch, "scratch"), _stream()))
+        _dev(scratch, "scratch"), int(nsplit), _stream()))
 
 
 def selective_scan_state_floats(inner: int, states: int, taps: int) -> int:
@@ -844,14 +847,15 @@ def conv_silu(x, taps, bias, positions, token_seq, cu_q, slots, state, states: i
 
 
 def dt_softplus(low, w, b, dt) -> None:
-    """dt = softplus(low[:, :rank] @ w.T + b) in float32; low rows may be a view."""
+    """dt = softplus(low[:, :rank] @ w + b) in float32, w [rank, inner] (the stored matrix transposed);
+    low rows may be a view."""
     _rows(low, "dt_softplus low")
     n, inner = dt.shape
-    rank = w.shape[1]
+    rank = w.shape[0]
     if low.dtype != torch.float32 or dt.dtype != torch.float32 or w.dtype != torch.float32 or b.dtype != torch.float32 \
-            or not dt.is_contiguous() or not w.is_contiguous() or tuple(w.shape) != (inner, rank) or b.numel() != inner \
+            or not dt.is_contiguous() or not w.is_contiguous() or tuple(w.shape) != (rank, inner) or b.numel() != inner \
             or low.shape[0] != n or low.shape[1] < rank:
-        raise KernelError("dt_softplus: float32 low [n, >= rank], w [inner, rank], b [inner], dt [n, inner]")
+        raise KernelError("dt_softplus: float32 low [n, >= rank], w [rank, inner], b [inner], dt [n, inner]")
     check(load().shk_dt_softplus(_dev(low, "low"), low.stride(0), _dev(w, "w"), _dev(b, "b"), rank, inner,
                                  _dev(dt, "dt"), n, _stream()))
 

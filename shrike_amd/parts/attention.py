@@ -298,7 +298,13 @@ class PagedAttention(Mixer):
                 plan.seq_name, plan.q0_name = f"attention_seq:{tag}", f"attention_q0:{tag}"
                 shape.add(plan.seq_name, seqs)
                 shape.add(plan.q0_name, q0)
-            shape.launch_key.append((key, "talking_mfma", shape.num_decode, plan.count))
+            if shape.num_decode:
+                # single tokens with many keys share them among workgroups: as many shares as bring the
+                # launch to twice the compute units, each worth 128 keys or more
+                reach = min(x for x in (s.window, s.chunk, shape.max_decode_ctx or 1) if x)
+                launched = shape.num_decode * hkv * -(-hkv * -(-(h // hkv) // 16) // 4)
+                plan.nsplit = max(1, min(2 * compute_units() // launched, reach // 128, 32))
+            shape.launch_key.append((key, "talking_mfma", shape.num_decode, plan.count, plan.nsplit))
             return
         if self.talking:
             # a token's heads stay together in one workgroup; single tokens with many keys share
@@ -372,14 +378,15 @@ class PagedAttention(Mixer):
                                "(the step function calls prepare() on every part)")
         q = qkv[:, : h * d]
         if plan.kernel == "talking_mfma":
-            floats = ops.attention_talking_mfma_scratch_floats(q.shape[0], h, hkv, self.value_dim)
+            floats = ops.attention_talking_mfma_scratch_floats(q.shape[0], h, hkv, self.value_dim, ctx.num_decode,
+                                                               plan.nsplit)
             scratch = ctx.buffer("attn_talking_sums", (floats,), torch.float32)
             ops.attention_talking_mfma(q, out, ctx.num_decode, h, hkv, d, self.value_dim, ctx.positions, ctx.token_seq,
                                        ctx.cu_q, ctx.extras[plan.seq_name] if plan.count else None,
                                        ctx.extras[plan.q0_name] if plan.count else None, plan.count, tables,
                                        cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale, scratch,
                                        chunk=s.chunk, r1=self.r1, r2=self.r2, talk=self.talk,
-                                       sink=getattr(s, "fixed_sink", None))
+                                       sink=getattr(s, "fixed_sink", None), nsplit=plan.nsplit)
             return
         if self.talking:
             floats = ops.attention_talking_scratch_floats(q.shape[0], h, self.value_dim, plan.nsplit)

@@ -51,8 +51,9 @@ class SelectiveScan(Mixer):
         s = self.spec
         if min(s.inner, s.state, s.dt_rank, s.conv) < 1:
             raise ValueError(f"{self.name}: inner, state, dt_rank and conv must be positive")
-        if s.state > 512 or s.conv > 64:
-            raise ValueError(f"{self.name}: at most 512 states a channel and 64 taps, got {s.state} and {s.conv}")
+        if s.state > 512 or s.conv > 64 or s.dt_rank > 1024:
+            raise ValueError(f"{self.name}: at most 512 states a channel, 64 taps and a step-size rank of 1024, got "
+                             f"{s.state}, {s.conv} and {s.dt_rank}")
         if ops.selective_scan_state_floats(s.inner, s.state, s.conv) != self.state_floats():
             raise RuntimeError(f"{self.name}: the kernel's state layout and the cache's size disagree")
 
@@ -61,7 +62,7 @@ class SelectiveScan(Mixer):
         self.taps = tensors[self._t("conv")].contiguous()
         self.conv_bias = tensors[self._t("conv.b")].contiguous()
         self.w_x = runtime.weight(tensors[self._t("x")])
-        self.w_dt = tensors[self._t("dt")].contiguous()
+        self.w_dt = tensors[self._t("dt")].t().contiguous()  # [dt_rank, inner]: channels are neighbours in memory
         self.dt_bias = tensors[self._t("dt.b")].contiguous()
         self.a_log = tensors[self._t("A_log")].contiguous()
         self.skip = tensors[self._t("D")].contiguous()

@@ -308,6 +308,7 @@ def run_scan_chain(ops, uz, low_of, w, inner, states, rank, taps, dtype, state, 
     rows; low_of(x) gives W_x's float32 output for conv outputs x (the test's own product)."""
     got = {s: torch.zeros(uz[s].shape[0], inner, dtype=dtype, device="cuda") for s in uz}
     wd = {k: dev(v) for k, v in w.items()}
+    wd["dt"] = dev(w["dt"].t())  # the step-size matrix goes in transposed
     for step in plan:
         starts, lens = [st for _, _, st, _ in step], [c for _, _, _, c in step]
         positions, token_seq, cu = step_arrays(starts, lens)
@@ -519,7 +520,7 @@ def test_experts_products_against_the_plain_form(ops, dtype, n, width, ff, exper
 
 # ------------------------------------------------------------------ the same on the matrix units (bfloat16)
 
-def run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, scale, page_size, sink=0.0):
+def run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, scale, page_size, sink=0.0, nsplit=1):
     """seqs: {name: (q, k, v)}; steps: lists of (name, start, count), single tokens first.  Every
     sequence's keys and values are in the cache beforehand."""
     dtype = torch.bfloat16
@@ -552,12 +553,12 @@ def run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, scale, 
         rows = dev(torch.cat([seqs[s][0][st:st + c].reshape(c, H * D) for s, st, c in step]), dtype)
         n = rows.shape[0]
         out = torch.empty(n, H * V, dtype=dtype, device="cuda")
-        scratch = torch.empty(ops.attention_talking_mfma_scratch_floats(n, H, G, V), device="cuda")
+        scratch = torch.empty(ops.attention_talking_mfma_scratch_floats(n, H, G, V, single, nsplit), device="cuda")
         ops.attention_talking_mfma(rows, out, single, H, G, D, V, positions, token_seq, cu,
                                    i32(tile_seq) if tile_seq else None, i32(tile_q0) if tile_q0 else None, len(tile_seq),
                                    i32([table_of[s] for s, _, _ in step]), k_pool, v_pool, page_size, window, scale, scratch,
                                    r1=None if r1 is None else dev(r1), r2=None if r2 is None else dev(r2),
-                                   talk=None if talk is None else dev(talk), sink=sink)
+                                   talk=None if talk is None else dev(talk), sink=sink, nsplit=nsplit)
         at = 0
         for s, st, c in step:
             got[s][st:st + c] = out[at:at + c]
@@ -593,9 +594,10 @@ def test_mixed_head_attention_on_the_matrix_units(ops, H, G, D, V, window, page_
         [("a", 58, 1), ("d", 33, 1), ("b", 4, 33)],
         [("d", 34, 36), ("a", 59, 91)],                         # portions only, far into their sequences
     ]
-    got = run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, 0.3, page_size)
-    for s, n in lens.items():
-        close(got[s], want[s].reshape(n, H * V), dtype, f"sequence {s}", tol=2e-2)
+    for nsplit in (1, 3):  # (single tokens' keys in one workgroup, or shared among three)
+        got = run_talking_mfma(ops, seqs, steps, H, G, D, V, r1, r2, talk, window, 0.3, page_size, nsplit=nsplit)
+        for s, n in lens.items():
+            close(got[s], want[s].reshape(n, H * V), dtype, f"sequence {s}, {nsplit} shares", tol=2e-2)
 
 
 @pytest.mark.parametrize("cuts", ["whole", "decode"])
@@ -612,7 +614,8 @@ def test_the_window_ends_where_it_should_on_the_matrix_units(ops, cuts):
         r1, r2 = torch.tensor([0.5, 0.0]), torch.tensor([1.0, 3.0])
         talk = torch.tensor([[1.0, 0.0], [0.25, 0.75]])
         steps = [[("s", 0, n)]] if cuts == "whole" else [[("s", 0, target + 1)]] + [[("s", t, 1)] for t in range(target + 1, n)]
-        got = run_talking_mfma(ops, {"s": (q, k, v)}, steps, H, G, D, V, r1, r2, talk, window, 1.0, page_size)["s"].float().cpu()
+        got = run_talking_mfma(ops, {"s": (q, k, v)}, steps, H, G, D, V, r1, r2, talk, window, 1.0, page_size,
+                               nsplit=1 if cuts == "whole" else 4)["s"].float().cpu()
         seen = got[:, 0].abs() > 30.0
         want = torch.zeros(n, dtype=torch.bool)
         want[target:min(n, target + window)] = True
