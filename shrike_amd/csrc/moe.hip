@@ -354,6 +354,126 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same two products for lists of many pairs, tiled through LDS: a workgroup forms 128 pairs x 128
+// weight rows (gate/up: 64 features of each; down: 128 columns) in steps of 32 along k.  The four
+// wavefronts (2 x 2) take 64 x 64 each: four A and four B operands from LDS feed sixteen matrix
+// instructions.  Rows of 32 elements lie 80 bytes apart in LDS, so the sixteen 16-byte reads of an
+// operand meet every bank once.  The next step's pieces are fetched into registers while this one is
+// multiplied.  Sums run over k in the same order as in the kernels above: the same bits.
+constexpr int kTileRows = 128;
+constexpr int kTileLd = 40;  // elements between rows in LDS (32 and 16 bytes of padding)
+
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+    moe_tiled_mfma_kernel(const bf16* __restrict__ a, const int32_t* __restrict__ order,
+                          const int32_t* __restrict__ counts, const bf16* __restrict__ w0, const bf16* __restrict__ w1,
+                          bf16* __restrict__ act_out, float* __restrict__ pair_out, int n, int k, int m, int top, int act) {
+  __shared__ __attribute__((aligned(16))) uint16_t sa[2][kTileRows * kTileLd];
+  __shared__ __attribute__((aligned(16))) uint16_t sb[2][kTileRows * kTileLd];
+  const int e = blockIdx.z;
+  const int count = min(counts[e], n);
+  const int row0 = blockIdx.y * kTileRows;
+  if (row0 >= count) return;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int i = lane % 16, kg = lane / 16;
+  const int wm = wave / 2, wn = wave % 2;
+  const int lr = tid / 4, lp = tid % 4;  // the row (and the one 64 below) and the 16-byte piece that this thread stages
+  const int32_t* list = order + static_cast<size_t>(e) * n;
+  const bf16* arow[2];
+  const bf16* brow[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = row0 + lr + 64 * h;
+    const int pair = r < count ? list[r] : -1;
+    // gate/up: a pair's row is its token's; down: its own row of activations
+    arow[h] = pair < 0 ? nullptr : a + static_cast<size_t>(GATED ? min(pair / top, n - 1) : min(pair, n * top - 1)) * k + lp * 8;
+    if (GATED) {
+      const int f = blockIdx.x * 64 + lr;
+      brow[h] = f < m ? (h == 0 ? w0 : w1) + (static_cast<size_t>(e) * m + f) * k + lp * 8 : nullptr;
+    } else {
+      const int c = blockIdx.x * 128 + lr + 64 * h;
+      brow[h] = c < m ? w0 + (static_cast<size_t>(e) * m + c) * k + lp * 8 : nullptr;
+    }
+  }
+  uint4 ra[2], rb[2];
+  auto fetch = [&](int k0) {
+    const bool have = k0 + lp * 8 < k;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      ra[h] = rb[h] = make_uint4(0, 0, 0, 0);
+      if (have && arow[h]) ra[h] = *reinterpret_cast<const uint4*>(arow[h] + k0);
+      if (have && brow[h]) rb[h] = *reinterpret_cast<const uint4*>(brow[h] + k0);
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      *reinterpret_cast<uint4*>(&sa[buf][(lr + 64 * h) * kTileLd + lp * 8]) = ra[h];
+      *reinterpret_cast<uint4*>(&sb[buf][(lr + 64 * h) * kTileLd + lp * 8]) = rb[h];
+    }
+  };
+  mf32x4 acc[4][4];
+#pragma unroll
+  for (int am = 0; am < 4; ++am)
+#pragma unroll
+    for (int bn = 0; bn < 4; ++bn) acc[am][bn] = mf32x4{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < k; k0 += 32, buf ^= 1) {
+    const bool more = k0 + 32 < k;
+    if (more) fetch(k0 + 32);
+    mbf16x8 af[4], bf[4];
+#pragma unroll
+    for (int am = 0; am < 4; ++am)
+      af[am] = __builtin_bit_cast(mbf16x8, *reinterpret_cast<const uint4*>(&sa[buf][(wm * 64 + am * 16 + i) * kTileLd + kg * 8]));
+#pragma unroll
+    for (int bn = 0; bn < 4; ++bn) {
+      // gate/up: operands 0, 1 are this wavefront's 32 gate features, 2, 3 the same features of up (rows 64 on)
+      const int brw = GATED ? (bn / 2) * 64 + wn * 32 + (bn % 2) * 16 + i : wn * 64 + bn * 16 + i;
+      bf[bn] = __builtin_bit_cast(mbf16x8, *reinterpret_cast<const uint4*>(&sb[buf][brw * kTileLd + kg * 8]));
+    }
+#pragma unroll
+    for (int am = 0; am < 4; ++am)
+#pragma unroll
+      for (int bn = 0; bn < 4; ++bn)
+        acc[am][bn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[bn], af[am], acc[am][bn], 0, 0, 0);
+    if (more) stage(buf ^ 1);
+    __syncthreads();
+  }
+  // this lane holds weight rows 4 kg + r of operand bn for the pair in row wm * 64 + am * 16 + i of the tile
+#pragma unroll
+  for (int am = 0; am < 4; ++am) {
+    const int r = row0 + wm * 64 + am * 16 + i;
+    if (r >= count) continue;
+    const int pair = min(max(list[r], 0), n * top - 1);
+    if (GATED) {
+      bf16* dst = act_out + static_cast<size_t>(pair) * m;
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn) {
+        const int f = blockIdx.x * 64 + wn * 32 + bn * 16 + 4 * kg;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (f + q < m) dst[f + q] = from_float<bf16>(gate_act(acc[am][bn][q], act) * acc[am][bn + 2][q]);
+      }
+    } else {
+      float* dst = pair_out + static_cast<size_t>(pair) * m;
+#pragma unroll
+      for (int bn = 0; bn < 4; ++bn) {
+        const int c = blockIdx.x * 128 + wn * 64 + bn * 16 + 4 * kg;
+        if (c + 3 < m) {
+          *reinterpret_cast<float4*>(dst + c) = make_float4(acc[am][bn][0], acc[am][bn][1], acc[am][bn][2], acc[am][bn][3]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (c + q < m) dst[c + q] = acc[am][bn][q];
+        }
+      }
+    }
+  }
+}
+
 // out[t, c] = add[t, c] + sum_k weights[t, k] * pair_out[t * top + k, c], k in the order chosen
 __global__ void __launch_bounds__(256)
     moe_join_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, const bf16* __restrict__ add,
@@ -445,12 +565,23 @@ extern "C" int shk_moe_experts_grouped(const void* x, const int32_t* chosen, con
   const long long ints = static_cast<long long>(experts) * n + experts;
   float* pair_out = reinterpret_cast<float*>(static_cast<char*>(scratch) + ((ints * 4 + 15) / 16) * 16);
   moe_lists_kernel<<<experts, 256, 0, s>>>(chosen, n, top, order, counts);
-  const int row_tiles = (n + 31) / 32;
-  moe_gate_up_mfma_kernel<<<dim3((ff + 127) / 128, row_tiles, experts), 256, 0, s>>>(
-      static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
-      static_cast<bf16*>(act_buf), n, width, ff, top, act);
-  moe_down_mfma_kernel<<<dim3((width + 255) / 256, row_tiles, experts), 256, 0, s>>>(
-      static_cast<const bf16*>(act_buf), order, counts, static_cast<const bf16*>(w_down), pair_out, n, width, ff, top);
+  if (static_cast<long long>(n) * top >= 64LL * experts) {
+    // lists of 64 pairs and more on average: tiles of 128 pairs through LDS
+    const int row_tiles = (n + kTileRows - 1) / kTileRows;
+    moe_tiled_mfma_kernel<true><<<dim3((ff + 63) / 64, row_tiles, experts), 256, 0, s>>>(
+        static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
+        static_cast<bf16*>(act_buf), nullptr, n, width, ff, top, act);
+    moe_tiled_mfma_kernel<false><<<dim3((width + 127) / 128, row_tiles, experts), 256, 0, s>>>(
+        static_cast<const bf16*>(act_buf), order, counts, static_cast<const bf16*>(w_down), nullptr, nullptr, pair_out, n,
+        ff, width, top, act);
+  } else {
+    const int row_tiles = (n + 31) / 32;
+    moe_gate_up_mfma_kernel<<<dim3((ff + 127) / 128, row_tiles, experts), 256, 0, s>>>(
+        static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
+        static_cast<bf16*>(act_buf), n, width, ff, top, act);
+    moe_down_mfma_kernel<<<dim3((width + 255) / 256, row_tiles, experts), 256, 0, s>>>(
+        static_cast<const bf16*>(act_buf), order, counts, static_cast<const bf16*>(w_down), pair_out, n, width, ff, top);
+  }
   moe_join_kernel<<<dim3((width + 255) / 256, n), 256, 0, s>>>(pair_out, weights, static_cast<const bf16*>(add),
                                                                static_cast<bf16*>(out), width, top);
   SHK_LAUNCH_CHECK("moe_experts_grouped");

@@ -59,11 +59,12 @@ __global__ void __launch_bounds__(256)
   y[static_cast<size_t>(t) * inner + c] = from_float<T>(silu_f(acc));
 }
 
-constexpr int kDtTokens = 8;  // tokens a workgroup: the matrix is read once for all of them
+constexpr int kDtTokens = 8;  // tokens a workgroup where a step has many: the matrix is read once for all of them
 
 // dt[t, c] = softplus(b[c] + sum_r W[r, c] * low[t, r]) in float32; W is given transposed, [rank, inner], so
 // that neighbouring channels' weights are neighbours in memory.  A token's sum runs over r in ascending
 // order whatever else is in the step.
+template <int kDtTokens>
 __global__ void __launch_bounds__(256)
     dt_softplus_kernel(const float* __restrict__ low, int ld, const float* __restrict__ wt, const float* __restrict__ b,
                        int rank, int inner, float* __restrict__ dt, int n) {
@@ -78,7 +79,8 @@ __global__ void __launch_bounds__(256)
   float acc[kDtTokens];
 #pragma unroll
   for (int k = 0; k < kDtTokens; ++k) acc[k] = b[c];
-  for (int r = 0; r < rank; ++r) {
+#pragma unroll 8
+  for (int r = 0; r < rank; ++r) {  // (eight rows' loads on their way at once)
     const float w = wt[static_cast<size_t>(r) * inner + c];
 #pragma unroll
     for (int k = 0; k < kDtTokens; ++k)
@@ -351,9 +353,16 @@ extern "C" int shk_dt_softplus(const float* low, int ld, const float* w, const f
               n, inner, rank);
   if (n == 0) return 0;
   SHK_REQUIRE(low && w && b && dt, "dt_softplus: null pointer");
-  dim3 grid((inner + 255) / 256, (n + kDtTokens - 1) / kDtTokens);
-  dt_softplus_kernel<<<grid, 256, kDtTokens * rank * sizeof(float), static_cast<hipStream_t>(stream)>>>(
-      low, ld, w, b, rank, inner, dt, n);
+  if (n <= 32) {
+    // few tokens: a wavefront per (64 channels, token), so that the launch has workgroups enough
+    SHK_REQUIRE(n <= 65535, "dt_softplus: bad n");
+    dt_softplus_kernel<1><<<dim3((inner + 63) / 64, n), 64, rank * sizeof(float), static_cast<hipStream_t>(stream)>>>(
+        low, ld, w, b, rank, inner, dt, n);
+  } else {
+    dim3 grid((inner + 255) / 256, (n + kDtTokens - 1) / kDtTokens);
+    dt_softplus_kernel<kDtTokens><<<grid, 256, kDtTokens * rank * sizeof(float), static_cast<hipStream_t>(stream)>>>(
+        low, ld, w, b, rank, inner, dt, n);
+  }
   SHK_LAUNCH_CHECK("dt_softplus");
   return 0;
 }

@@ -938,12 +938,12 @@ def moe_route(logits, correction, top: int, chosen, weights) -> None:
                                _dev(chosen, "chosen"), _dev(weights, "weights"), n, _stream()))
 
 
-MOE_GROUPED_FROM = 4  # tokens of a step from which the experts' products run per expert on the matrix units
+MOE_GROUPED_FROM = 1  # tokens of a step from which the experts' products run per expert on the matrix units
 
 
 def moe_grouped(n: int, width: int, ff: int, dtype) -> bool:
     """Whether a step of n tokens runs its experts' products per expert on the matrix units:
-    bfloat16, rows in multiples of 8 elements, and enough tokens that experts are shared."""
+    bfloat16 and rows in multiples of 8 elements."""
     return dtype == torch.bfloat16 and n >= MOE_GROUPED_FROM and width % 8 == 0 and ff % 8 == 0
 
 

@@ -624,7 +624,9 @@ def test_the_window_ends_where_it_should_on_the_matrix_units(ops, cuts):
 
 @pytest.mark.parametrize("n, width, ff, experts, top, shared", [(4, 64, 24, 5, 2, True), (7, 104, 32, 4, 4, False),
                                                                 (40, 128, 64, 8, 1, True), (130, 72, 40, 9, 3, False),
-                                                                (300, 256, 96, 6, 2, True), (33, 64, 8, 70, 6, False)])
+                                                                (300, 256, 96, 6, 2, True), (33, 64, 8, 70, 6, False),
+                                                                (200, 104, 72, 3, 2, False), (1, 64, 24, 5, 2, True),
+                                                                (520, 136, 200, 2, 2, True)])
 def test_experts_products_per_expert_on_the_matrix_units(ops, n, width, ff, experts, top, shared):
     dtype = torch.bfloat16
     assert ops.moe_grouped(n, width, ff, dtype)
