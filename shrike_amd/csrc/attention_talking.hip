@@ -318,36 +318,72 @@ __global__ void __launch_bounds__(256)
   const int slab = key_slab(head_dim);
   const size_t k_head = static_cast<size_t>(page_size) * head_dim;  // elements of a page's head
   const size_t v_head = static_cast<size_t>(page_size) * v_dim;
+  // the pages of a chunk's keys: this lane's two keys as A rows of the scores, and its 8 keys of the values
+  auto pages_of = [&](int j0, int (&kp)[2], int& vp) {
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const int jk = j0 + 8 * (i / 4) + 4 * t2 + i % 4;
+      kp[t2] = -1;
+      if (jk >= lo_min && jk <= pos_max) {
+        const int page = table[jk / page_size];
+        kp[t2] = page >= 0 && page < num_pages ? page : -1;
+      }
+    }
+    const int jg = j0 + 8 * kg;
+    vp = -1;
+    if (jg + 7 >= lo_min && jg <= pos_max) {
+      const int page = table[jg / page_size];
+      vp = page >= 0 && page < num_pages ? page : -1;
+    }
+  };
+  int kpage[2], vpage;
+  pages_of(j_begin, kpage, vpage);
   for (int j0 = j_begin; j0 <= j_end; j0 += 32) {
-    // scores: A row m of product t2 is the key j0 + 8 (m / 4) + 4 t2 + m % 4
+    // All of the chunk's operands are asked for before anything is multiplied, and the next chunk's
+    // pages are looked up meanwhile: a chunk waits for memory once.
+    // keys: A row m of product t2 is the key j0 + 8 (m / 4) + 4 t2 + m % 4
+    uint4 kf[2][KS];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const int jk = j0 + 8 * (i / 4) + 4 * t2 + i % 4;
+      const bf16* kr = k_pool + (static_cast<size_t>(max(kpage[t2], 0)) * kv_heads + ck) * k_head;
+      const int slot = jk % page_size;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        kf[t2][ks] = make_uint4(0, 0, 0, 0);
+        const int e = ks * 32 + kg * 8;
+        if (kpage[t2] >= 0 && e < head_dim)
+          kf[t2][ks] = *reinterpret_cast<const uint4*>(kr + (static_cast<size_t>(e / slab) * page_size + slot) * slab + e % slab);
+      }
+    }
+    // values: A row i of block b is value element (b % vb) * 16 + i of key/value head cv0 + b / vb, keys jg .. + 8
+    const int jg = j0 + 8 * kg;
+    union VFrag {
+      uint4 u;
+      uint16_t h[8];
+    } vf[NB];
+    {
+      const int slot = jg % page_size;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const int cvl = b / vb, d = (b % vb) * 16 + i;
+        vf[b].u = make_uint4(0, 0, 0, 0);
+        if (cvl < cvn && vpage >= 0 && d < v_dim)
+          vf[b].u = *reinterpret_cast<const uint4*>(v_pool + (static_cast<size_t>(vpage) * kv_heads + cv0 + cvl) * v_head +
+                                                    static_cast<size_t>(d) * page_size + slot);
+      }
+    }
+    const int vpage_now = vpage;
+    if (j0 + 32 <= j_end) pages_of(j0 + 32, kpage, vpage);
     tf32x4 s[2];
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
       s[t2] = tf32x4{0.f, 0.f, 0.f, 0.f};
-      const int jk = j0 + 8 * (i / 4) + 4 * t2 + i % 4;
-      int page = -1;
-      if (jk >= lo_min && jk <= pos_max) {
-        page = table[jk / page_size];
-        if (page < 0 || page >= num_pages) page = -1;
-      }
-      const bf16* kr = k_pool + (static_cast<size_t>(max(page, 0)) * kv_heads + ck) * k_head;
-      const int slot = jk % page_size;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        uint4 kv = make_uint4(0, 0, 0, 0);
-        const int e = ks * 32 + kg * 8;
-        if (page >= 0 && e < head_dim)
-          kv = *reinterpret_cast<const uint4*>(kr + (static_cast<size_t>(e / slab) * page_size + slot) * slab + e % slab);
-        s[t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, kv), qf[ks], s[t2], 0, 0, 0);
-      }
+      for (int ks = 0; ks < KS; ++ks)
+        s[t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, kf[t2][ks]), qf[ks], s[t2], 0, 0, 0);
     }
-    // this lane: the scores of keys j0 + 8 kg + 4 t2 + r for its row i; their page (8 aligned keys share one)
-    const int jg = j0 + 8 * kg;
-    int vpage = -1;
-    if (jg + 7 >= lo_min && jg <= pos_max) {
-      vpage = table[jg / page_size];
-      if (vpage < 0 || vpage >= num_pages) vpage = -1;
-    }
+    // this lane: the scores of keys jg + 4 t2 + r for its row i (8 aligned keys share a page)
     float x[8];
     float mx = -INFINITY;
 #pragma unroll
@@ -357,7 +393,7 @@ __global__ void __launch_bounds__(256)
         const int j = jg + 4 * t2 + r;
         float v = s[t2][r] * scale_l2;
         if (r1) v -= bias1 * __log2f(1.f + bias2 * static_cast<float>(pos - j));
-        const bool seen = vpage >= 0 && j >= lo && j <= pos;
+        const bool seen = vpage_now >= 0 && j >= lo && j <= pos;
         v = seen ? v : -INFINITY;
         x[4 * t2 + r] = v;
         mx = fmaxf(mx, v);
@@ -384,28 +420,17 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[b][r] *= alpha;
     }
-    // values: A row i of block b is value element (b % vb) * 16 + i of key/value head cv0 + b / vb, keys jg .. + 8
-    const int slot = jg % page_size;
+    const bool ragged = jg < lo_min || jg + 7 > pos_max;  // keys that no row of the tile reads may hold anything
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      const int cvl = b / vb, d = (b % vb) * 16 + i;
-      union {
-        uint4 u;
-        uint16_t h[8];
-      } vf;
-      vf.u = make_uint4(0, 0, 0, 0);
-      if (cvl < cvn) {
-        if (vpage >= 0 && d < v_dim) {
-          vf.u = *reinterpret_cast<const uint4*>(v_pool + (static_cast<size_t>(vpage) * kv_heads + cv0 + cvl) * v_head +
-                                                 static_cast<size_t>(d) * page_size + slot);
-          if (jg < lo_min || jg + 7 > pos_max) {  // keys that no row of the tile reads may hold anything
+      if (b / vb < cvn) {
+        if (ragged) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (jg + e < lo_min || jg + e > pos_max) vf.h[e] = 0;
-          }
+          for (int e = 0; e < 8; ++e)
+            if (jg + e < lo_min || jg + e > pos_max) vf[b].h[e] = 0;
         }
-        o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, vf.u), __builtin_bit_cast(tbf16x8, pf.u),
-                                                       o[b], 0, 0, 0);
+        o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, vf[b].u),
+                                                       __builtin_bit_cast(tbf16x8, pf.u), o[b], 0, 0, 0);
       }
     }
   }

@@ -79,23 +79,28 @@ __global__ void __launch_bounds__(256)
   float acc[kDtTokens];
 #pragma unroll
   for (int k = 0; k < kDtTokens; ++k) acc[k] = b[c];
-#pragma unroll 8
-  for (int r = 0; r < rank; ++r) {  // (eight rows' loads on their way at once)
-    const float w = wt[static_cast<size_t>(r) * inner + c];
+  for (int r0 = 0; r0 < rank; r0 += 8) {  // eight rows' weights on their way at once
+    float w[8];
 #pragma unroll
-    for (int k = 0; k < kDtTokens; ++k)
-      if (k < count) acc[k] = fmaf(w, lows[k * rank + r], acc[k]);
+    for (int u = 0; u < 8; ++u) w[u] = r0 + u < rank ? wt[static_cast<size_t>(r0 + u) * inner + c] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (r0 + u >= rank) break;
+#pragma unroll
+      for (int k = 0; k < kDtTokens; ++k)
+        if (k < count) acc[k] = fmaf(w[u], lows[k * rank + r0 + u], acc[k]);
+    }
   }
 #pragma unroll
   for (int k = 0; k < kDtTokens; ++k)
     if (k < count) dt[static_cast<size_t>(t0 + k) * inner + c] = softplus_f(acc[k]);
 }
 
-constexpr int kStatesPerLane = 8;
+constexpr int kStatesPerLane = 4;
 constexpr int kScanBlock = 16;  // tokens whose inputs are fetched together
 
 // One sequence's tokens for a block of channels.  LANES lanes share a channel's states
-// (LANES * 8 >= states); a wavefront holds 64 / LANES channels.
+// (LANES * 4 >= states); a wavefront holds 64 / LANES channels.
 template <typename T, int LANES>
 __global__ void __launch_bounds__(256)
     selective_scan_kernel(const float* __restrict__ dt, const T* __restrict__ x, const float* __restrict__ bc,
@@ -219,7 +224,7 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-constexpr int kRowsPerLane = 16;
+constexpr int kRowsPerLane = 8;
 constexpr int kRetBlock = 8;  // tokens whose inputs are fetched together
 
 // the heads that the columns of one workgroup (256 / lanes of them) can belong to
@@ -230,7 +235,7 @@ inline int retention_heads_a_workgroup(int lanes, int heads, int v_dim) {
 }
 
 // One sequence's tokens for one (head, value column); LANES lanes share the column's rows
-// of S (LANES * 16 >= dim).
+// of S (LANES * 8 >= dim).
 template <int LANES>
 __global__ void __launch_bounds__(256)
     retention_scan_kernel(const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
