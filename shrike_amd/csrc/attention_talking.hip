@@ -481,10 +481,48 @@ __global__ void __launch_bounds__(256)
   u_out[(static_cast<size_t>(t) * heads + head) * gv + rest] = den > 0.f ? val / den : 0.f;
 }
 
-// out[t, h, d] = sum_g talk[h, g] * U[t, g, c(h), d]   (talk null: U[t, h, c(h), d])
+// out[t, h, d] = sum_g talk[h, g] * U[t, g, c(h), d]   (talk null: U[t, h, c(h), d]).  A thread takes one
+// value element of one key/value head and forms it for all query heads of that key/value head, eight
+// at a time: what it reads of U serves them all.
 __global__ void __launch_bounds__(256)
     talking_mix_kernel(const float* __restrict__ u_in, const float* __restrict__ talk, bf16* __restrict__ out, int heads,
                        int kv_heads, int v_dim) {
+  const int t = blockIdx.y;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= kv_heads * v_dim) return;
+  const int c = idx / v_dim, d = idx % v_dim;
+  const int group = heads / kv_heads;
+  const size_t gv = static_cast<size_t>(kv_heads) * v_dim;
+  const float* ut = u_in + static_cast<size_t>(t) * heads * gv + idx;
+  bf16* ot = out + static_cast<size_t>(t) * heads * v_dim + d;
+  if (!talk) {
+    for (int k = 0; k < group; ++k) {
+      const int h = c * group + k;
+      ot[static_cast<size_t>(h) * v_dim] = from_float<bf16>(ut[h * gv]);
+    }
+    return;
+  }
+  for (int k0 = 0; k0 < group; k0 += 8) {
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+    const float* row = talk + static_cast<size_t>(c * group + k0) * heads;
+    for (int g = 0; g < heads; ++g) {
+      const float u = ut[g * gv];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (k0 + k < group) acc[k] = fmaf(row[k * heads + g], u, acc[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (k0 + k < group) ot[static_cast<size_t>(c * group + k0 + k) * v_dim] = from_float<bf16>(acc[k]);
+  }
+}
+
+// The same a thread per output element, for steps of few tokens (more workgroups than the kernel above has).
+__global__ void __launch_bounds__(256)
+    talking_mix_each_kernel(const float* __restrict__ u_in, const float* __restrict__ talk, bf16* __restrict__ out,
+                            int heads, int kv_heads, int v_dim) {
   const int t = blockIdx.y;
   const int o = blockIdx.x * blockDim.x + threadIdx.x;
   if (o >= heads * v_dim) return;
@@ -666,9 +704,15 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
 #undef SHK_KS
 #undef SHK_NB
 #undef SHK_GO
-  const int outs = heads * v_dim;
-  talking_mix_kernel<<<dim3((outs + 255) / 256, n), 256, 0, s>>>(scratch, talk, static_cast<bf16*>(out), heads, kv_heads,
-                                                                v_dim);
+  if (n >= 64) {
+    const int outs = kv_heads * v_dim;
+    talking_mix_kernel<<<dim3((outs + 255) / 256, n), 256, 0, s>>>(scratch, talk, static_cast<bf16*>(out), heads,
+                                                                  kv_heads, v_dim);
+  } else {
+    const int outs = heads * v_dim;
+    talking_mix_each_kernel<<<dim3((outs + 255) / 256, n), 256, 0, s>>>(scratch, talk, static_cast<bf16*>(out), heads,
+                                                                       kv_heads, v_dim);
+  }
   SHK_LAUNCH_CHECK("attention_talking_bf16");
   return 0;
 }

@@ -105,16 +105,30 @@ __global__ void __launch_bounds__(kLnThreads)
     __syncthreads();
     row_moments(d, hidden, deps, scratch, mean, inv);
   }
-  for (int c = threadIdx.x; c < hidden; c += kLnThreads) {
+  // With few rows a row's columns are shared among gridDim.y workgroups (each forms the addend's
+  // moments for itself).  The entries that are only read are fetched four at a time; the sum runs
+  // over j in ascending order either way.
+  const int per = (hidden + gridDim.y - 1) / gridDim.y;
+  const int c_end = min(hidden, static_cast<int>(blockIdx.y + 1) * per);
+  const int reads = delta ? count - 1 : count;
+  for (int c = blockIdx.y * per + threadIdx.x; c < c_end; c += kLnThreads) {
+    const float* base = history + row * hidden + c;
     float acc = 0.f;
-    for (int j = 0; j < count; ++j) {
-      float* at = history + j * stride + row * hidden + c;
-      float v = *at;
-      if (delta && j == count - 1) {
-        v += (d[c] - mean) * inv * dweight[c] + (dbias ? dbias[c] : 0.f);
-        *at = v;
-      }
-      acc = fmaf(coef[j], v, acc);
+    int j = 0;
+    for (; j + 4 <= reads; j += 4) {
+      const float v0 = base[j * stride], v1 = base[(j + 1) * stride], v2 = base[(j + 2) * stride],
+                  v3 = base[(j + 3) * stride];
+      acc = fmaf(coef[j], v0, acc);
+      acc = fmaf(coef[j + 1], v1, acc);
+      acc = fmaf(coef[j + 2], v2, acc);
+      acc = fmaf(coef[j + 3], v3, acc);
+    }
+    for (; j < reads; ++j) acc = fmaf(coef[j], base[j * stride], acc);
+    if (delta) {
+      float* at = history + (count - 1) * stride + row * hidden + c;
+      const float v = *at + ((d[c] - mean) * inv * dweight[c] + (dbias ? dbias[c] : 0.f));
+      *at = v;
+      acc = fmaf(coef[count - 1], v, acc);
     }
     out[row * hidden + c] = acc;
   }
@@ -170,11 +184,12 @@ extern "C" int shk_mix_history(float* history, long long stride, const float* co
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t lds = static_cast<size_t>(hidden) * sizeof(float);
   const size_t split_stride = static_cast<size_t>(n) * hidden;
+  const dim3 grid(n, n < 64 && hidden >= 8 * kLnThreads ? 8 : 1);
   if (dtype == kF32)
-    mix_history_kernel<float><<<n, kLnThreads, lds, s>>>(history, static_cast<size_t>(stride), coef, count, out, hidden,
+    mix_history_kernel<float><<<grid, kLnThreads, lds, s>>>(history, static_cast<size_t>(stride), coef, count, out, hidden,
                                                          delta, delta_splits, split_stride, dweight, dbias, deps);
   else
-    mix_history_kernel<bf16><<<n, kLnThreads, lds, s>>>(history, static_cast<size_t>(stride), coef, count, out, hidden,
+    mix_history_kernel<bf16><<<grid, kLnThreads, lds, s>>>(history, static_cast<size_t>(stride), coef, count, out, hidden,
                                                         delta, delta_splits, split_stride, dweight, dbias, deps);
   SHK_LAUNCH_CHECK("mix_history");
   return 0;

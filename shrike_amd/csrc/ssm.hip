@@ -21,6 +21,25 @@
 namespace shk {
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+
+// Sum over the LANES neighbouring lanes that share a channel or a column (LANES a power of two; every
+// lane of the group gets it).  Up to 16 lanes meet by lane permutations of the vector unit: within
+// fours [1,0,3,2] and [2,3,0,1], then mirrored halves of 8 and of 16 (all lanes of a four already
+// hold the four's sum, so its mirror image holds the other four's).
+template <int CTRL>
+__device__ __forceinline__ float dpp_moved(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+  if (LANES >= 2) v += dpp_moved<0xB1>(v);
+  if (LANES >= 4) v += dpp_moved<0x4E>(v);
+  if (LANES >= 8) v += dpp_moved<0x141>(v);
+  if (LANES >= 16) v += dpp_moved<0x140>(v);
+  if (LANES >= 32) v += __shfl_xor(v, 16, kWave);
+  if (LANES >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
 // y[t, c] = silu(bias[c] + sum_k taps[c, K - 1 - k] * x(t - k, c)): x(t - k) is a row of this
@@ -96,12 +115,12 @@ __global__ void __launch_bounds__(256)
     if (k < count) dt[static_cast<size_t>(t0 + k) * inner + c] = softplus_f(acc[k]);
 }
 
-constexpr int kStatesPerLane = 4;
+constexpr int kStatesPerLane = 4;  // (8 where a channel has more than 256 states)
 constexpr int kScanBlock = 16;  // tokens whose inputs are fetched together
 
 // One sequence's tokens for a block of channels.  LANES lanes share a channel's states
 // (LANES * 4 >= states); a wavefront holds 64 / LANES channels.
-template <typename T, int LANES>
+template <typename T, int LANES, int kStatesPerLane>
 __global__ void __launch_bounds__(256)
     selective_scan_kernel(const float* __restrict__ dt, const T* __restrict__ x, const float* __restrict__ bc,
                           int ld_bc, int b_off, int c_off, const T* __restrict__ z, int ldz,
@@ -159,12 +178,13 @@ __global__ void __launch_bounds__(256)
       for (int i = 0; i < kStatesPerLane; ++i) {
         const int n = part * kStatesPerLane + i;
         if (n < states) {
-          S[i] = fmaf(expf(step * A[i]), S[i], dx * bt[n]);
+          // (bfloat16 models: the hardware's exponential, float32 all the same; float32 models: the library's)
+          const float decay = sizeof(T) == 2 ? __expf(step * A[i]) : expf(step * A[i]);
+          S[i] = fmaf(decay, S[i], dx * bt[n]);
           y = fmaf(S[i], ct[n], y);
         }
       }
-#pragma unroll
-      for (int off = LANES / 2; off > 0; off >>= 1) y += __shfl_xor(y, off, kWave);
+      y = group_sum<LANES>(y);
       if (part == 0 && active) {
         y = fmaf(dc, xv, y);
         out[static_cast<size_t>(t0 + k) * inner + c] = from_float<T>(y * silu_f(gs[k]));
@@ -224,7 +244,7 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-constexpr int kRowsPerLane = 8;
+constexpr int kRowsPerLane = 8;  // (16 where a head has more than 512 elements)
 constexpr int kRetBlock = 8;  // tokens whose inputs are fetched together
 
 // the heads that the columns of one workgroup (256 / lanes of them) can belong to
@@ -236,7 +256,7 @@ inline int retention_heads_a_workgroup(int lanes, int heads, int v_dim) {
 
 // One sequence's tokens for one (head, value column); LANES lanes share the column's rows
 // of S (LANES * 8 >= dim).
-template <int LANES>
+template <int LANES, int kRowsPerLane>
 __global__ void __launch_bounds__(256)
     retention_scan_kernel(const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
                           const float* __restrict__ decay, int heads, int dim, int v_dim,
@@ -298,8 +318,7 @@ __global__ void __launch_bounds__(256)
           o = fmaf(S[i], qt[d], o);
         }
       }
-#pragma unroll
-      for (int off = LANES / 2; off > 0; off >>= 1) o += __shfl_xor(o, off, kWave);
+      o = group_sum<LANES>(o);
       if (part == 0 && active) out[static_cast<size_t>(t0 + k) * heads * v_dim + unit] = o;
     }
   }
@@ -378,7 +397,7 @@ extern "C" int shk_selective_scan(const float* dt, const void* x, const float* b
                                   const int32_t* cu_q, const int32_t* slots, float* state, long long slot_stride,
                                   void* out, int dtype, int num_seqs, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "selective_scan: unknown dtype %d", dtype);
-  SHK_REQUIRE(num_seqs >= 0 && inner > 0 && states > 0 && states <= 64 * kStatesPerLane && num_taps >= 1,
+  SHK_REQUIRE(num_seqs >= 0 && inner > 0 && states > 0 && states <= 512 && num_taps >= 1,
               "selective_scan: bad sizes seqs=%d inner=%d states=%d", num_seqs, inner, states);
   SHK_REQUIRE(b_off >= 0 && c_off >= 0 && b_off + states <= ld_bc && c_off + states <= ld_bc && ldz >= inner &&
                   ld_raw >= inner,
@@ -390,10 +409,10 @@ extern "C" int shk_selective_scan(const float* dt, const void* x, const float* b
   SHK_REQUIRE(dt && x && bc && z && a_log && dskip && raw && positions && cu_q && slots && state && out,
               "selective_scan: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int lanes = lanes_for(states, kStatesPerLane);
+  const int lanes = states > 64 * kStatesPerLane ? 64 : lanes_for(states, kStatesPerLane);
 #define SHK_GO(T, L)                                                                                                 \
-  selective_scan_kernel<T, L><<<dim3((inner + 256 / L - 1) / (256 / L), num_seqs), 256,                              \
-                                kScanBlock * 2 * states * sizeof(float), s>>>(                                       \
+  selective_scan_kernel<T, L, (L == 64 ? 8 : kStatesPerLane)>                                                        \
+      <<<dim3((inner + 256 / L - 1) / (256 / L), num_seqs), 256, kScanBlock * 2 * states * sizeof(float), s>>>(      \
       dt, static_cast<const T*>(x), bc, ld_bc, b_off, c_off, static_cast<const T*>(z), ldz, a_log, dskip, inner,     \
       states, num_taps, static_cast<const T*>(raw), ld_raw, positions, cu_q, slots, state, slot_stride,              \
       static_cast<T*>(out))
@@ -440,7 +459,7 @@ extern "C" int shk_retention_scan(const float* proj, int ld, int q_off, int k_of
                                   int num_seqs, int heads, int dim, int v_dim, const int32_t* positions,
                                   const int32_t* cu_q, const int32_t* slots, float* state, long long slot_stride,
                                   float* out, void* stream) {
-  SHK_REQUIRE(num_seqs >= 0 && heads > 0 && dim > 0 && dim <= 64 * kRowsPerLane && v_dim > 0,
+  SHK_REQUIRE(num_seqs >= 0 && heads > 0 && dim > 0 && dim <= 1024 && v_dim > 0,
               "retention_scan: bad sizes seqs=%d heads=%d dim=%d v_dim=%d", num_seqs, heads, dim, v_dim);
   SHK_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= ld && k_off + heads * dim <= ld &&
                   v_off + heads * v_dim <= ld,
@@ -451,7 +470,7 @@ extern "C" int shk_retention_scan(const float* proj, int ld, int q_off, int k_of
   SHK_REQUIRE(num_seqs <= 65535, "retention_scan: at most 65535 sequences a call");
   SHK_REQUIRE(proj && decay && positions && cu_q && slots && state && out, "retention_scan: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int lanes = lanes_for(dim, kRowsPerLane);
+  const int lanes = dim > 64 * kRowsPerLane ? 64 : lanes_for(dim, kRowsPerLane);
   const int units = heads * v_dim;
   const size_t a_token = static_cast<size_t>(retention_heads_a_workgroup(lanes, heads, v_dim)) * 2 * dim * sizeof(float);
   SHK_REQUIRE(a_token <= 64000, "retention_scan: %d heads of %d elements a workgroup do not fit its LDS",
@@ -459,7 +478,7 @@ extern "C" int shk_retention_scan(const float* proj, int ld, int q_off, int k_of
   const int block = static_cast<int>(64000 / a_token) < kRetBlock ? static_cast<int>(64000 / a_token) : kRetBlock;
   const size_t lds = block * a_token;
 #define SHK_GO(L)                                                                                              \
-  retention_scan_kernel<L><<<dim3((units + 256 / L - 1) / (256 / L), num_seqs), 256, lds, s>>>(                \
+  retention_scan_kernel<L, (L == 64 ? 16 : kRowsPerLane)><<<dim3((units + 256 / L - 1) / (256 / L), num_seqs), 256, lds, s>>>(                \
       proj, ld, q_off, k_off, v_off, decay, heads, dim, v_dim, positions, cu_q, slots, state, slot_stride, out, block)
   switch (lanes) {
     case 1: SHK_GO(1); break;

@@ -51,8 +51,8 @@ class SelectiveScan(Mixer):
         s = self.spec
         if min(s.inner, s.state, s.dt_rank, s.conv) < 1:
             raise ValueError(f"{self.name}: inner, state, dt_rank and conv must be positive")
-        if s.state > 256 or s.conv > 64 or s.dt_rank > 1024:
-            raise ValueError(f"{self.name}: at most 256 states a channel, 64 taps and a step-size rank of 1024, got "
+        if s.state > 512 or s.conv > 64 or s.dt_rank > 1024:
+            raise ValueError(f"{self.name}: at most 512 states a channel, 64 taps and a step-size rank of 1024, got "
                              f"{s.state}, {s.conv} and {s.dt_rank}")
         if ops.selective_scan_state_floats(s.inner, s.state, s.conv) != self.state_floats():
             raise RuntimeError(f"{self.name}: the kernel's state layout and the cache's size disagree")
@@ -126,8 +126,8 @@ class Retention(Mixer):
         s = self.spec
         if min(s.num_heads, s.head_dim, s.value_dim) < 1:
             raise ValueError(f"{self.name}: heads, head_dim and value_dim must be positive")
-        if s.head_dim > 512:
-            raise ValueError(f"{self.name}: head_dim {s.head_dim} is more than the 512 the scan kernel holds")
+        if s.head_dim > 1024:
+            raise ValueError(f"{self.name}: head_dim {s.head_dim} is more than the 1024 the scan kernel holds")
         if len(s.decay) != s.num_heads:
             raise ValueError(f"{self.name}: {len(s.decay)} decays for {s.num_heads} heads")
         if self.position is not None:

@@ -151,6 +151,7 @@ def test_default_model_dir_env_override(monkeypatch):
     assert reg.DEFAULT_MODEL_DIR == "/somewhere/else"
     monkeypatch.delenv("SHRIKE_MODEL_DIR")
     importlib.reload(reg)
+    import shrike_amd.models.ligipel as lg
     import shrike_amd.models.minilorn as n
     import shrike_amd.models.mofarax as m
     import shrike_amd.models.qwen2 as q
@@ -158,6 +159,7 @@ def test_default_model_dir_env_override(monkeypatch):
     importlib.reload(q)  # the reload emptied the registry; register again
     importlib.reload(m)
     importlib.reload(n)
+    importlib.reload(lg)
 
 
 def test_plugins_named_in_the_environment_are_loaded_for_an_unknown_architecture(tmp_path, monkeypatch):

@@ -332,7 +332,7 @@ def run_scan_chain(ops, uz, low_of, w, inner, states, rank, taps, dtype, state, 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("inner, states, rank, taps", [(40, 3, 2, 2), (96, 12, 5, 4), (50, 70, 7, 1), (72, 33, 9, 3),
-                                                       (300, 16, 30, 5)])
+                                                       (300, 16, 30, 5), (24, 300, 3, 2)])
 def test_selective_scan_in_pieces_and_in_used_slots(ops, dtype, inner, states, rank, taps):
     torch.manual_seed(inner)
     w = scan_weights(inner, states, rank, taps, inner + states)
@@ -400,7 +400,8 @@ def test_rotation_of_float32_rows(ops, heads, dim, rot, base):
     assert torch.equal(got[:, :off].cpu(), x[:, :off]) and torch.equal(got[:, off + heads * dim:].cpu(), x[:, off + heads * dim:])
 
 
-@pytest.mark.parametrize("heads, dim, v_dim", [(2, 16, 20), (3, 40, 16), (1, 12, 50), (2, 64, 64), (4, 128, 32)])
+@pytest.mark.parametrize("heads, dim, v_dim", [(2, 16, 20), (3, 40, 16), (1, 12, 50), (2, 64, 64), (4, 128, 32),
+                                               (1, 600, 8), (3, 8, 3)])
 def test_retention_scan_in_pieces_and_in_used_slots(ops, heads, dim, v_dim):
     torch.manual_seed(dim + v_dim)
     decay = torch.tensor([1.0, 0.5, 0.97, 0.999][:heads])
