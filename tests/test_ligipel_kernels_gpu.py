@@ -212,7 +212,7 @@ def test_a_key_that_stands_out_shows_where_the_window_ends(ops, cuts):
     holds the key, at a page border, a tile's border and far back."""
     H, G, D, V, page_size = 2, 1, 16, 4, 16
     n = 420
-    for target, window in [(15, 16), (16, 33), (63, 64), (64, 65), (3, 400), (130, 136), (200, 1)]:
+    for target, window in [(15, 16), (16, 33), (63, 64), (64, 65), (3, 400), (130, 141), (200, 1)]:
         g = torch.Generator().manual_seed(target)
         q = torch.randn(n, H, D, generator=g) * 0.1
         k = torch.randn(n, G, D, generator=g) * 0.1
@@ -451,7 +451,7 @@ def test_retention_keeps_a_far_key(ops):
 
 # ------------------------------------------------------------------ experts
 
-@pytest.mark.parametrize("experts, top", [(3, 3), (5, 2), (9, 1), (8, 4), (70, 6)])
+@pytest.mark.parametrize("experts, top", [(3, 3), (5, 2), (9, 1), (8, 3), (70, 6)])
 def test_router_choice_and_weights(ops, experts, top):
     torch.manual_seed(experts)
     n = 37
@@ -604,7 +604,7 @@ def test_mixed_head_attention_on_the_matrix_units(ops, H, G, D, V, window, page_
 @pytest.mark.parametrize("cuts", ["whole", "decode"])
 def test_the_window_ends_where_it_should_on_the_matrix_units(ops, cuts):
     H, G, D, V, page_size, n = 2, 1, 16, 16, 16, 300
-    for target, window in [(15, 16), (16, 33), (63, 64), (64, 65), (3, 290), (130, 136), (200, 1), (31, 32), (32, 1)]:
+    for target, window in [(15, 16), (16, 33), (63, 64), (64, 65), (3, 290), (130, 141), (200, 1), (31, 32), (32, 1)]:
         g = torch.Generator().manual_seed(target)
         q = torch.randn(n, H, D, generator=g) * 0.1
         k = torch.randn(n, G, D, generator=g) * 0.1
@@ -627,7 +627,7 @@ def test_the_window_ends_where_it_should_on_the_matrix_units(ops, cuts):
                                                                 (40, 128, 64, 8, 1, True), (130, 72, 40, 9, 3, False),
                                                                 (300, 256, 96, 6, 2, True), (33, 64, 8, 70, 6, False),
                                                                 (200, 104, 72, 3, 2, False), (1, 64, 24, 5, 2, True),
-                                                                (520, 136, 200, 2, 2, True)])
+                                                                (520, 152, 200, 2, 2, True)])
 def test_experts_products_per_expert_on_the_matrix_units(ops, n, width, ff, experts, top, shared):
     dtype = torch.bfloat16
     assert ops.moe_grouped(n, width, ff, dtype)

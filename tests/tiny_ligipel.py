@@ -70,7 +70,7 @@ LIG_B = {
 LIG_C = {
     "architecture": "Ligipel", "vocab": 300, "width": 128, "norm": {"eps": 2e-5}, "logit_scale": 1.5,
     "layers": [
-        _with(_parallel(_attn(4, 4, 64, 128, 300, scale=0.2), _scan(256, 16, 8, 4)), _moe(8, 2, 64, shared=96)),
+        _with(_parallel(_attn(4, 4, 64, 128, 300, scale=0.2), _scan(256, 16, 8, 4)), _moe(8, 2, 48, shared=80)),
         _with(_parallel(_attn(8, 2, 32, 32, 33), _scan(128, 8, 4, 3)), _moe(4, 1, 128)),
         _with(_retention(2, 64, 64, [0.98, 0.999], base=1.0e5, dims=32), _moe(8, 8, 32, shared=32)),
     ],
