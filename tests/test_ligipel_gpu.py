@@ -24,7 +24,8 @@ pytestmark = pytest.mark.gpu
 TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
 # lengths that end before, on and after the edges of the models' windows (7, 40; 1; 33, 300)
 # and of their pages
-LENGTHS = {"A": [1, 8, 49, 97, 130, 10], "B": [3, 41, 40, 29, 8, 150], "C": [2, 70, 33, 340]}
+LENGTHS = {"A": [1, 8, 49, 97, 130, 10], "B": [3, 41, 40, 29, 8, 150], "C": [2, 70, 33, 340], "D": [1, 90, 17, 2, 64],
+           "E": [16, 17, 80, 1, 33]}
 
 
 @pytest.fixture(scope="module")
@@ -49,7 +50,7 @@ def engine_parts(model_dir, dtype, page_size, pages, graphs=True, slots=4):
     return model, cache, ModelRunner(model, cache, rt, graphs=graphs)
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_the_stream_after_every_layer(name, model_root):
     """float32: what every layer hands on (after the depth average) against the plain
     model's, for a prompt that crosses window edges."""
@@ -83,7 +84,8 @@ def test_the_stream_after_every_layer(name, model_root):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name, page_size", [("A", 16), ("B", 4), ("B", 16), ("C", 32), ("A", 8), ("C", 16)])
+@pytest.mark.parametrize("name, page_size", [("A", 16), ("B", 4), ("B", 16), ("C", 32), ("A", 8), ("C", 16),
+                                             ("D", 16), ("E", 16), ("E", 8)])
 def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtype, model_root, tmp_path):
     model_dir = make_model_dir(name, model_root, dtype=dtype)
     vocab = CONFIGS[name]["vocab"]
@@ -104,7 +106,8 @@ def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtyp
     got = tb.collect(outputs)
     assert all(np.isfinite(rows).all() for rows in outputs.values()), "a page that nobody holds was read"
     reused = check_pages(tb.steps, read_pages(tmp_path / "out", tb.steps), page_size, mixed_budget // page_size)
-    assert reused > 0, "the pool was meant to be so small that pages are used again"
+    if any(layer["type"] == "parallel" for layer in CONFIGS[name]["layers"]):  # (retention alone keeps no pages)
+        assert reused > 0, "the pool was meant to be so small that pages are used again"
 
     scale = {rid: np.abs(w).max() for rid, w in want.items()}
     worst, over = {}, []

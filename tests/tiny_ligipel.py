@@ -76,9 +76,27 @@ LIG_C = {
     ],
 }
 
-CONFIGS = {"A": LIG_A, "B": LIG_B, "C": LIG_C}
-SEEDS = {"A": 5, "B": 13, "C": 29}
-PAGE_SIZES = {"A": 16, "B": 4, "C": 32}
+# retention only: a model without any paged cache
+LIG_D = {
+    "architecture": "Ligipel", "vocab": 120, "width": 48, "norm": {"eps": 1e-5}, "logit_softcap": 20.0,
+    "layers": [
+        _with(_retention(4, 8, 8, [0.75, 0.9, 0.96, 0.995], base=300.0, dims=8), _moe(4, 2, 16, shared=24)),
+        _with(_retention(2, 24, 12, [0.99, 0.6], base=7.0, dims=2), None),
+    ],
+}
+
+# side-by-side mixers only; as many key/value heads as heads; a window of exactly a page
+LIG_E = {
+    "architecture": "Ligipel", "vocab": 160, "width": 72, "norm": {"eps": 1e-5}, "logit_scale": 2.0,
+    "layers": [
+        _with(_parallel(_attn(3, 3, 40, 24, 16), _scan(64, 4, 3, 2)), _moe(3, 3, 24)),
+        _with(_parallel(_attn(5, 5, 8, 16, 17), _scan(80, 20, 6, 4)), _moe(7, 2, 8, shared=16)),
+    ],
+}
+
+CONFIGS = {"A": LIG_A, "B": LIG_B, "C": LIG_C, "D": LIG_D, "E": LIG_E}
+SEEDS = {"A": 5, "B": 13, "C": 29, "D": 41, "E": 53}
+PAGE_SIZES = {"A": 16, "B": 4, "C": 32, "D": 16, "E": 16}
 
 
 def make_model_dir(name: str, root=None, dtype: str = "float32", mode: str = "unit") -> Path:
