@@ -219,9 +219,10 @@ __global__ void __launch_bounds__(256)
 // results.  One pass over the keys, no weights in memory.
 //
 // A wavefront serves 16 query rows that share a sequence and a key/value head for the keys:
-// 16 consecutive tokens of a prompt's portion for one head (tile_seq / tile_q0 list them), or
-// one single token's heads of a key/value head.  Keys go by in chunks of 32, aligned to 32 in
-// the sequence:
+// one single token's heads of a key/value head (talking_mfma_kernel, operands straight from
+// memory), or 16 consecutive tokens of a prompt's portion for one head (talking_tiles_lds_kernel,
+// tile_seq / tile_q0 list the tiles; a workgroup's four heads share what it stages in LDS).  Keys
+// go by in chunks of 32, aligned to 32 in the sequence:
 //
 //   S^T = K Q^T   [32 keys x 16 rows]  two v_mfma_f32_16x16x32_bf16 per 32 elements of a head;
 //                 A = keys straight from their slabs (a lane's 8 elements are 16 bytes), and
@@ -253,9 +254,8 @@ __global__ void __launch_bounds__(256)
                         const int32_t* __restrict__ token_seq, const int32_t* __restrict__ tables, int table_stride,
                         const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool, int page_size, int num_pages,
                         int window, int chunk, float scale_l2, const float* __restrict__ r1,
-                        const float* __restrict__ r2, int has_sink, float sink_l2, const int32_t* __restrict__ cu_q,
-                        const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int tiles_mode,
-                        int nsplit, float* __restrict__ partial, int vh_pass) {
+                        const float* __restrict__ r2, int has_sink, float sink_l2, int nsplit,
+                        float* __restrict__ partial, int vh_pass) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int i = lane % 16, kg = lane / 16;
   const int group = heads / kv_heads;
@@ -264,25 +264,14 @@ __global__ void __launch_bounds__(256)
   const int cv0 = blockIdx.z * vh_pass;
   const int cvn = min(vh_pass, kv_heads - cv0);
   // the lane's query row
-  int t, head, seq, ck;
-  bool valid;
-  if (tiles_mode) {
-    if (unit >= heads) return;
-    seq = tile_seq[blockIdx.x];
-    t = cu_q[seq] + tile_q0[blockIdx.x] + i;
-    valid = t < cu_q[seq + 1];
-    head = unit;
-    ck = head / group;
-  } else {
-    const int subs = (group + 15) / 16;
-    if (unit >= kv_heads * subs) return;
-    t = blockIdx.x / nsplit;
-    seq = token_seq[t];
-    ck = unit / subs;
-    const int within = (unit % subs) * 16 + i;
-    valid = within < group;
-    head = ck * group + (valid ? within : 0);
-  }
+  const int subs = (group + 15) / 16;
+  if (unit >= kv_heads * subs) return;
+  const int t = blockIdx.x / nsplit;
+  const int seq = token_seq[t];
+  const int ck = unit / subs;
+  const int within = (unit % subs) * 16 + i;
+  const bool valid = within < group;
+  const int head = ck * group + (valid ? within : 0);
   const int pos = valid ? positions[t] : -1;
   const int lo = valid ? first_key(pos, window, chunk) : (1 << 30);
   int pos_max = pos, lo_min = lo;
@@ -308,7 +297,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
   for (int b = 0; b < NB; ++b) o[b] = tf32x4{0.f, 0.f, 0.f, 0.f};
   // single tokens with many keys: share `share` of nsplit takes a run of the chunks (the sink is the first one's)
-  const int share = tiles_mode ? 0 : blockIdx.x % nsplit;
+  const int share = blockIdx.x % nsplit;
   const int chunk_lo = lo_min / 32, chunk_hi = pos_max / 32;
   const int per_share = (chunk_hi - chunk_lo + nsplit) / nsplit;
   const int j_begin = (chunk_lo + share * per_share) * 32;
@@ -455,6 +444,220 @@ __global__ void __launch_bounds__(256)
     for (int r = 0; r < 4; ++r) {
       const int d = (b % vb) * 16 + 4 * kg + r;
       if (d < v_dim) dst[static_cast<size_t>(cv0 + cvl) * v_dim + d] = o[b][r] * inv;
+    }
+  }
+}
+
+// Prompt portions with a chunk staged once for four heads: a workgroup serves one tile of 16
+// queries, four query heads of one key/value head (a wavefront each) and a pass of key/value heads
+// for the values.  A chunk's 32 keys and the 32 values of every value element of the pass's
+// key/value heads are fetched once by the workgroup (the next chunk's pieces are on their way into
+// registers while this one is multiplied), laid into LDS (key rows 16 bytes longer than a head,
+// value rows of 32 keys 80 bytes apart: an operand's sixteen 16-byte reads meet every bank once),
+// and every wavefront takes its operands from there.  NB = key/value heads of a pass x blocks of 16
+// values, at most 16: with 64 registers of sums two workgroups share a compute unit.
+template <int KS, int NB>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+    talking_tiles_lds_kernel(const bf16* __restrict__ q, int q_stride, float* __restrict__ u_out, int heads, int kv_heads,
+                             int head_dim, int v_dim, const int32_t* __restrict__ positions,
+                             const int32_t* __restrict__ tables, int table_stride, const bf16* __restrict__ k_pool,
+                             const bf16* __restrict__ v_pool, int page_size, int num_pages, int window, int chunk,
+                             float scale_l2, const float* __restrict__ r1, const float* __restrict__ r2, int has_sink,
+                             float sink_l2, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ tile_seq,
+                             const int32_t* __restrict__ tile_q0, int vh_pass) {
+  constexpr int KLD = KS * 32 + 8;      // elements between key rows in LDS
+  constexpr int VLD = 40;               // elements between value rows (32 keys and 16 bytes)
+  constexpr int KPT = KS >= 2 ? KS / 2 : 1;  // 16-byte pieces of keys a thread stages: 32 keys x 4 KS pieces / 256
+  constexpr int VPT = NB >= 4 ? NB / 4 : 1;  // of values: NB x 16 rows x 4 pieces / 256
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds_t[];
+  uint16_t* sk = lds_t;                      // [32][KLD]
+  uint16_t* sv = lds_t + 32 * KLD;           // [NB * 16][VLD]
+  __shared__ int group_ok[4];                // whether the chunk's four groups of 8 keys have a page
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int i = lane % 16, kg = lane / 16;
+  const int group = heads / kv_heads;
+  const int quads = (group + 3) / 4;
+  const int ck = blockIdx.y / quads;
+  const int within = (blockIdx.y % quads) * 4 + wave;
+  const bool has_head = within < group;
+  const int head = ck * group + (has_head ? within : 0);
+  const int vb = (v_dim + 15) / 16;
+  const int cv0 = blockIdx.z * vh_pass;
+  const int cvn = min(vh_pass, kv_heads - cv0);
+  const int seq = tile_seq[blockIdx.x];
+  const int t = cu_q[seq] + tile_q0[blockIdx.x] + i;
+  const bool valid = t < cu_q[seq + 1];
+  const int pos = valid ? positions[t] : -1;
+  const int lo = valid ? first_key(pos, window, chunk) : (1 << 30);
+  int pos_max = pos, lo_min = lo;
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) {
+    pos_max = max(pos_max, __shfl_xor(pos_max, off, kWave));
+    lo_min = min(lo_min, __shfl_xor(lo_min, off, kWave));
+  }
+  if (pos_max < 0) return;  // (the same for all four wavefronts: they serve the same tokens)
+  const int32_t* table = tables + static_cast<size_t>(seq) * table_stride;
+  const float bias1 = r1 ? r1[head] : 0.f, bias2 = r1 ? r2[head] : 0.f;
+  tbf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    const int e = ks * 32 + kg * 8;
+    if (valid && has_head && e < head_dim)
+      v = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(t) * q_stride + head * head_dim + e);
+    qf[ks] = __builtin_bit_cast(tbf16x8, v);
+  }
+  tf32x4 o[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) o[b] = tf32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = has_sink ? sink_l2 : -INFINITY;
+  float l_run = has_sink ? 1.f : 0.f;
+  const int slab = key_slab(head_dim);
+  const size_t k_head = static_cast<size_t>(page_size) * head_dim;
+  const size_t v_head = static_cast<size_t>(page_size) * v_dim;
+  const int kpieces = head_dim / 8;         // 16-byte pieces of a key
+  const int vrows = cvn * v_dim;            // value rows of a chunk: (key/value head of the pass, element)
+  union Piece {
+    uint4 u;
+    uint16_t h[8];
+  };
+  Piece rk[KPT], rv[VPT];
+  int rv_ok[VPT];
+  auto page_at = [&](int j) {
+    const int page = table[j / page_size];
+    return page >= 0 && page < num_pages ? page : -1;
+  };
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int r = 0; r < KPT; ++r) {
+      const int p = tid + 256 * r;
+      const int key = p / kpieces, e = (p % kpieces) * 8;
+      const int j = j0 + key;
+      rk[r].u = make_uint4(0, 0, 0, 0);
+      if (key < 32 && j >= lo_min && j <= pos_max) {
+        const int page = page_at(j);
+        if (page >= 0)
+          rk[r].u = *reinterpret_cast<const uint4*>(k_pool + (static_cast<size_t>(page) * kv_heads + ck) * k_head +
+                                                    (static_cast<size_t>(e / slab) * page_size + j % page_size) * slab +
+                                                    e % slab);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < VPT; ++r) {
+      const int p = tid + 256 * r;
+      const int row = p / 4, jg = j0 + 8 * (p % 4);  // row = key/value head of the pass * v_dim + element
+      rv[r].u = make_uint4(0, 0, 0, 0);
+      rv_ok[r] = 0;
+      if (row < vrows && jg + 7 >= lo_min && jg <= pos_max) {
+        const int page = page_at(jg);
+        if (page >= 0) {
+          rv_ok[r] = 1;
+          rv[r].u = *reinterpret_cast<const uint4*>(v_pool + (static_cast<size_t>(page) * kv_heads + cv0 + row / v_dim) * v_head +
+                                                    static_cast<size_t>(row % v_dim) * page_size + jg % page_size);
+          if (jg < lo_min || jg + 7 > pos_max) {  // keys that no row of the tile reads may hold anything
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (jg + e < lo_min || jg + e > pos_max) rv[r].h[e] = 0;
+          }
+        }
+      }
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int r = 0; r < KPT; ++r) {
+      const int p = tid + 256 * r;
+      const int key = p / kpieces, e = (p % kpieces) * 8;
+      if (key < 32) *reinterpret_cast<uint4*>(&sk[key * KLD + e]) = rk[r].u;
+    }
+#pragma unroll
+    for (int r = 0; r < VPT; ++r) {
+      const int p = tid + 256 * r;
+      const int row = p / 4, kq = p % 4;
+      if (row < vrows) {
+        // LDS rows go by blocks of 16 elements of a key/value head: block (cv * vb + d / 16), row d % 16
+        const int cv = row / v_dim, d = row % v_dim;
+        *reinterpret_cast<uint4*>(&sv[((cv * vb + d / 16) * 16 + d % 16) * VLD + kq * 8]) = rv[r].u;
+        if (row == 0) group_ok[kq] = rv_ok[r];
+      }
+    }
+  };
+  // (elements of a key beyond head_dim, and value rows beyond v_dim, are never staged: they stay zero from here)
+  for (int z = tid; z < (32 * KLD + NB * 16 * VLD) / 2; z += 256) reinterpret_cast<uint32_t*>(lds_t)[z] = 0u;
+  const int j_begin = lo_min / 32 * 32;
+  fetch(j_begin);
+  for (int j0 = j_begin; j0 <= pos_max; j0 += 32) {
+    __syncthreads();  // (the chunk before has been read; the first time: the zeros are in place)
+    stage();
+    __syncthreads();
+    if (j0 + 32 <= pos_max) fetch(j0 + 32);
+    if (!has_head) continue;
+    tf32x4 s[2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      s[t2] = tf32x4{0.f, 0.f, 0.f, 0.f};
+      const int key = 8 * (i / 4) + 4 * t2 + i % 4;  // A row i of product t2
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const uint4 kv = *reinterpret_cast<const uint4*>(&sk[key * KLD + ks * 32 + kg * 8]);
+        s[t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, kv), qf[ks], s[t2], 0, 0, 0);
+      }
+    }
+    const int jg = j0 + 8 * kg;
+    const bool paged = group_ok[kg] != 0;
+    float x[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int j = jg + 4 * t2 + r;
+        float v = s[t2][r] * scale_l2;
+        if (r1) v -= bias1 * __log2f(1.f + bias2 * static_cast<float>(pos - j));
+        const bool seen = paged && j >= lo && j <= pos;
+        v = seen ? v : -INFINITY;
+        x[4 * t2 + r] = v;
+        mx = fmaxf(mx, v);
+      }
+    const float m_new = fmaxf(m_run, rows_max(mx));
+    const float alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_new) : 0.f;
+    float psum = 0.f;
+    Piece pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float p = x[e] > -INFINITY ? __builtin_amdgcn_exp2f(x[e] - m_new) : 0.f;
+      psum += p;
+      const bf16 pb = from_float<bf16>(p);
+      pf.h[e] = __builtin_bit_cast(uint16_t, pb);
+    }
+    l_run = l_run * alpha + rows_sum(psum);
+    m_run = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[b][r] *= alpha;
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (b < cvn * vb) {
+        const uint4 vv = *reinterpret_cast<const uint4*>(&sv[(b * 16 + i) * VLD + kg * 8]);
+        o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tbf16x8, vv), __builtin_bit_cast(tbf16x8, pf.u),
+                                                       o[b], 0, 0, 0);
+      }
+    }
+  }
+  if (!valid || !has_head) return;
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  float* dst = u_out + (static_cast<size_t>(t) * heads + head) * kv_heads * v_dim;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (b >= cvn * vb) continue;
+    const int cv = cv0 + b / vb;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int d = (b % vb) * 16 + 4 * kg + r;
+      if (d < v_dim) dst[static_cast<size_t>(cv) * v_dim + d] = o[b][r] * inv;
     }
   }
 }
@@ -621,13 +824,10 @@ static void launch_talking_mfma(dim3 grid, hipStream_t s, const bf16* q, int q_s
                                 int head_dim, int v_dim, const int32_t* positions, const int32_t* token_seq,
                                 const int32_t* tables, int table_stride, const bf16* k_pool, const bf16* v_pool,
                                 int page_size, int num_pages, int window, int chunk, float scale_l2, const float* r1,
-                                const float* r2, int has_sink, float sink_l2, const int32_t* cu_q,
-                                const int32_t* tile_seq, const int32_t* tile_q0, int tiles_mode, int nsplit,
-                                float* partial, int vh_pass) {
+                                const float* r2, int has_sink, float sink_l2, int nsplit, float* partial, int vh_pass) {
   talking_mfma_kernel<KS, NB><<<grid, 256, 0, s>>>(q, q_stride, u, heads, kv_heads, head_dim, v_dim, positions, token_seq,
                                                    tables, table_stride, k_pool, v_pool, page_size, num_pages, window,
-                                                   chunk, scale_l2, r1, r2, has_sink, sink_l2, cu_q, tile_seq, tile_q0,
-                                                   tiles_mode, nsplit, partial, vh_pass);
+                                                   chunk, scale_l2, r1, r2, has_sink, sink_l2, nsplit, partial, vh_pass);
 }
 
 }  // namespace shk
@@ -670,7 +870,7 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
   launch_talking_mfma<KS, NB>(grid, s, static_cast<const bf16*>(q), q_stride, scratch, heads, kv_heads, head_dim, v_dim, \
                               positions, token_seq, tables, table_stride, static_cast<const bf16*>(k_pool),             \
                               static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale * log2e, r1,  \
-                              r2, has_sink, sink * log2e, cu_q, tile_seq, tile_q0, mode, shares, partial, vh_pass)
+                              r2, has_sink, sink * log2e, shares, partial, vh_pass)
 #define SHK_NB(KS)                                                                                                     \
   if (nb <= 2) SHK_GO(KS, 2);                                                                                          \
   else if (nb <= 4) SHK_GO(KS, 4);                                                                                     \
@@ -683,7 +883,7 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
   else { SHK_NB(8); }
   if (num_single > 0) {
     // single tokens: a key/value head's query heads are a tile's rows; one value head a workgroup
-    const int mode = 0, vh_pass = 1, nb = vb, shares = nsplit;
+    const int vh_pass = 1, nb = vb, shares = nsplit;
     const int units = kv_heads * ((group + 15) / 16);
     dim3 grid(num_single * nsplit, (units + 3) / 4, kv_heads);
     SHK_KS()
@@ -694,12 +894,25 @@ extern "C" int shk_attention_talking_bf16(const void* q, int q_stride, void* out
     }
   }
   if (num_tiles > 0) {
-    // (8 blocks of sums a pass where a head's values allow it: two wavefronts then share a SIMD's registers)
-    const int mode = 1, shares = 1;
-    const int vh_pass = max(1, min(kv_heads, 8 / vb));
+    // a chunk staged once for four heads; 16 blocks of sums a pass where a head's values allow it
+    const int vh_pass = max(1, min(kv_heads, 16 / vb));
     const int nb = vh_pass * vb;
-    dim3 grid(num_tiles, (heads + 3) / 4, (kv_heads + vh_pass - 1) / vh_pass);
-    SHK_KS()
+    dim3 grid(num_tiles, kv_heads * ((group + 3) / 4), (kv_heads + vh_pass - 1) / vh_pass);
+#define SHK_LDS(KS, NB)                                                                                                \
+  talking_tiles_lds_kernel<KS, NB><<<grid, 256, (32 * (KS * 32 + 8) + NB * 16 * 40) * sizeof(uint16_t), s>>>(           \
+      static_cast<const bf16*>(q), q_stride, scratch, heads, kv_heads, head_dim, v_dim, positions, tables, table_stride, \
+      static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk,           \
+      scale * log2e, r1, r2, has_sink, sink * log2e, cu_q, tile_seq, tile_q0, vh_pass)
+#define SHK_LDS_NB(KS)                                                                                                 \
+  if (nb <= 4) SHK_LDS(KS, 4);                                                                                         \
+  else if (nb <= 8) SHK_LDS(KS, 8);                                                                                    \
+  else SHK_LDS(KS, 16)
+    if (ks <= 1) { SHK_LDS_NB(1); }
+    else if (ks <= 2) { SHK_LDS_NB(2); }
+    else if (ks <= 4) { SHK_LDS_NB(4); }
+    else { SHK_LDS_NB(8); }
+#undef SHK_LDS_NB
+#undef SHK_LDS
   }
 #undef SHK_KS
 #undef SHK_NB
