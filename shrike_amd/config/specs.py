@@ -83,6 +83,18 @@ class AttentionSpec:
     score (no tensor) in every head's denominator.  ``talking_heads``: a learned [heads, heads]
     matrix T mixes the softmax weights across heads, w_h = sum_g T[h, g] p_g, before head h
     applies them to the values of its own key/value head (the sink's share is not mixed).
+    ``qk_norm`` = (eps, weighted): every head of the queries and of the keys is divided by
+    sqrt(mean(x^2) + eps) after the projection (queries before their temperature); with
+    `weighted` also multiplied by a learned weight of the head's size that all heads share (one
+    for the queries, one for the keys).  ``bucket_bias`` = (rows, reach): a learned table [rows,
+    heads] whose row bucket(i - j) is added to the (capped) score of head h; the first rows // 2
+    rows stand for one distance each, the others are spread evenly over ln(distance) up to
+    `reach`, and the last row serves every distance beyond (parts/attention.py:
+    distance_buckets); rows None: as many as the file's tensor has.  ``shared_kv``: the layer has no key and value projections (and none of
+    their norms' weights); it reads the cache of another run (ScheduleEntry.cache_of) with its
+    own queries and mask.  ``cache_window``: what the layer's cache keeps where that is not its
+    own window, because a run that reads this cache looks further back ("own": the window;
+    None: everything).
     """
 
     kind: ClassVar[str] = "paged_attention"
@@ -105,6 +117,10 @@ class AttentionSpec:
     distance_bias: bool = False
     fixed_sink: float | None = None
     talking_heads: bool = False
+    qk_norm: tuple | None = None
+    bucket_bias: tuple | None = None
+    shared_kv: bool = False
+    cache_window: object = "own"
 
 
 @dataclass(frozen=True)
@@ -120,7 +136,8 @@ class LatentAttentionSpec:
     rot_theta ** (-2i / rotated), for the first ``rotated`` elements of the part (None: all
     of it; the rest pass unchanged).  Both norms are RMS norms with a weight and ``eps``.
     ``window`` / ``chunk`` bound the keys as in AttentionSpec.  Only c and the rotated key
-    part are cached."""
+    part are cached.  ``output_gate``: the heads' outputs side by side are multiplied by
+    sigmoid(W_g x) before the output matrix."""
 
     kind: ClassVar[str] = "latent_attention"
     num_heads: int
@@ -136,6 +153,7 @@ class LatentAttentionSpec:
     chunk: int | None = None
     names: Names = ()
     rotated: int | None = None
+    output_gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -214,8 +232,12 @@ class MoESpec:
     ``expert_size`` features.  Router logits W_router x in float32; scores = softmax over all
     experts; the ``top`` experts with the largest score + correction (a tensor of one number
     per expert, with ``correction``) are chosen; their weights are their scores over the
-    chosen ones' sum (+ 1e-20).  ``shared_size``: a gated expert of that many features that
-    every token passes and whose output is added (None: none)."""
+    chosen ones' sum (+ 1e-20), which is the softmax over the chosen experts' logits alone.
+    ``shared_size``: an expert of that many features that every token passes and whose output is
+    added (None: none).  ``gated`` False: experts (the shared one too) are down(act(up x)) and
+    have no gate matrix; their activation is then "relu_squared".  ``router_bias``: a learned
+    number per expert is added to the logits (a tensor).  ``shared_gate``: the shared expert's
+    output is multiplied by sigmoid(w . x), one number per token (a tensor [1, width])."""
 
     kind: ClassVar[str] = "moe"
     experts: int
@@ -225,6 +247,9 @@ class MoESpec:
     correction: bool = True
     activation: str = "silu"
     names: Names = ()
+    gated: bool = True
+    router_bias: bool = False
+    shared_gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -241,13 +266,18 @@ class DenseFFNSpec:
 
 @dataclass(frozen=True)
 class SwiGLUSpec:
-    """down(act(gate(x)) * up(x)) without biases; act is "silu" (SwiGLU proper) or
-    "gelu_tanh" (the tanh form of GELU)."""
+    """down(act(gate(x)) * up(x)) without biases; act is "silu" (SwiGLU proper),
+    "gelu_tanh" (the tanh form of GELU) or "quick_gelu" (g * sigmoid(1.702 g)).  With
+    ``limit`` the gate is bounded from above, g <- min(g, limit), and the other factor from
+    both sides, u <- clamp(u, -limit, limit), before the activation; ``up_shift`` is added to
+    that factor: down(act(g) * (u + up_shift))."""
 
     kind: ClassVar[str] = "swiglu"
     intermediate_size: int
     activation: str = "silu"
     names: Names = ()
+    limit: float | None = None
+    up_shift: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -309,6 +339,30 @@ class SandwichBlockSpec:
     mixer_post_name: str = "norm1b"
     ffn_norm_name: str = "norm2"
     ffn_post_name: str = "norm2b"
+
+
+@dataclass(frozen=True)
+class PostNormBlockSpec:
+    """The norm stands after the sum, and the stream is what the norm leaves:
+    x <- mixer_norm(alpha * x + s1 * mixer(x)); x <- ffn_norm(alpha * x + s2 * ffn(x)), the
+    sublayers reading x itself.  ``layer_scale``: s1 and s2 are learned vectors of the model's
+    width (tensors ``mixer_scale_name`` / ``ffn_scale_name`` below the block's name); else ones.
+    ``ffn`` may be None: the layer then has no feed-forward, no second norm and no second scale."""
+
+    kind: ClassVar[str] = "postnorm_residual"
+    name: str
+    mixer: object
+    ffn: object
+    mixer_norm: object
+    ffn_norm: object = None
+    alpha: float = 1.0
+    layer_scale: bool = False
+    mixer_name: str = "mix"
+    ffn_name: str = "mlp"
+    mixer_norm_name: str = "norm1"
+    ffn_norm_name: str = "norm2"
+    mixer_scale_name: str = "ls1"
+    ffn_scale_name: str = "ls2"
 
 
 @dataclass(frozen=True)

@@ -72,8 +72,24 @@ int shk_add_rmsnorm(float* resid, const void* delta, const float* weight, float 
                     int delta_splits, int resid_rows, void* stream);
 
 // out[i, j] = act(gu[i, j]) * gu[i, inter + j] for j < inter; gu is [n, 2*inter].
-// act 1: SiLU; act 2: GELU in its tanh form.
-int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act, void* stream);
+// act 1: SiLU; act 2: GELU in its tanh form; act 3: ReLU; act 4: g * sigmoid(1.702 g).  With limit > 0
+// the gate is bounded from above, g <- min(g, limit), and the other factor from both sides, before
+// anything else; up_shift is added to that factor: out = act(g) * (u + up_shift).
+int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act, float limit, float up_shift,
+                void* stream);
+
+// A stream that is normed after every sum (postnorm.hip): resid[r, :] <- (x / sqrt(mean(x^2) + eps)) *
+// weight with x = alpha * resid[r, :] + lscale * delta[r, :] (lscale float32 [hidden] or null: ones);
+// delta has `dtype`, or is float32 partial sums [delta_splits][n][hidden] added in order.  cast (of
+// `dtype`, or null) receives the new rows too.
+int shk_postnorm(float* resid, const void* delta, int delta_splits, float alpha, const float* lscale,
+                 const float* weight, float eps, void* cast, int dtype, int n, int hidden, void* stream);
+// dst[i] = src[i] in `dtype`.
+int shk_cast_rows(const float* src, void* dst, int dtype, long long numel, void* stream);
+// out = act(x) elementwise: 1 SiLU, 2 GELU (tanh form), 3 ReLU, 4 the square of ReLU.
+int shk_activate(const void* x, void* out, int dtype, long long numel, int act, void* stream);
+// out = x * sigmoid(gate) elementwise.
+int shk_gate_mul(const void* x, const void* gate, void* out, int dtype, long long numel, void* stream);
 
 // out[n, m] (+)= a[n, k] @ w[m, k]^T + bias[m].  a and w have in_dtype, out has
 // out_dtype, bias is float32 or null.  lda/ldo are row strides in elements.
@@ -148,12 +164,14 @@ int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int 
 // out is [n, heads * v_dim].  Softmax and accumulation are float32.  v_dim is the size of
 // a value (the value pool is [num_pages, kv_heads, v_dim, page_size]); softcap > 0 caps
 // the scaled scores, s <- softcap * tanh(s / softcap); sinks (float32 [heads] or null)
-// adds exp(sinks[head]) to the softmax's denominator, a term without key or value.
+// adds exp(sinks[head]) to the softmax's denominator, a term without key or value; dist_bias (float32
+// [heads, bias_rows] or null) adds dist_bias[head, min(p - j, bias_rows - 1)] to the score after the cap.
 int shk_attention(const void* q, int q_stride, void* out, int dtype, int n, int heads,
                   int kv_heads, int head_dim, const int32_t* positions, const int32_t* token_seq,
                   const int32_t* tables, int table_stride, int num_seqs, const void* k_pool,
                   const void* v_pool, int page_size, int num_pages, int window, int chunk, float scale,
-                  int v_dim, float softcap, const float* sinks, void* stream);
+                  int v_dim, float softcap, const float* sinks, const float* dist_bias, int bias_rows,
+                  void* stream);
 
 // Cache write for attention without rotation.  qkv is [n, heads * head_dim + kv_heads *
 // (head_dim + v_dim)]: queries, keys, values.  q_every > 0: the queries of the token at
@@ -161,8 +179,12 @@ int shk_attention(const void* q, int q_stride, void* out, int dtype, int n, int 
 // v_eps > 0: each head's value is divided by sqrt(mean(v^2) + v_eps) before it is stored.
 // Keys and values go to their page slots in the layouts of shk_rope_kv_store (values
 // [num_pages, kv_heads, v_dim, page_size]); write_kv 0 leaves the pools alone.
+// qk_eps > 0: every head of the queries and of the keys is divided by sqrt(mean(x^2) + qk_eps) first
+// and multiplied by q_weight / k_weight (float32 [head_dim], shared by the heads; null: none).
+// has_kv 0: qkv is [n, heads * head_dim], queries alone (a layer that reads another's cache).
 int shk_qkv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int head_dim, int v_dim,
-                  float q_coef, int q_every, float v_eps, const int32_t* positions,
+                  float q_coef, int q_every, float v_eps, float qk_eps, const float* q_weight,
+                  const float* k_weight, int has_kv, const int32_t* positions,
                   const int32_t* token_seq, const int32_t* tables, int table_stride, void* k_pool,
                   void* v_pool, int page_size, int num_pages, int write_kv, void* stream);
 
@@ -368,19 +390,22 @@ int shk_retention_scan(const float* proj, int ld, int q_off, int k_off, int v_of
 // their weights [n, top] are their scores over the chosen ones' sum (+ 1e-20).
 // shk_moe_experts: out[t] = add[t] (null: nothing) + sum_k weights[t, k] * W_down_e (act(W_gate_e
 // x_t) * (W_up_e x_t)), e = chosen[t, k]; matrices stacked row-major [experts, ff, width] and
-// [experts, width, ff]; act_buf [n * top, ff]; all of `dtype`; act 1 SiLU, 2 GELU (tanh form).
+// [experts, width, ff]; act_buf [n * top, ff]; all of `dtype`; act 1 SiLU, 2 GELU (tanh form), 3 ReLU
+// (experts without a gate whose activation is the square of ReLU pass their one matrix as both).
+// add_gate (float32, one number per token, gate_ld apart; null: none): add[t] is multiplied by
+// sigmoid(add_gate[t * gate_ld]).
 int shk_moe_route(const float* logits, int ld, const float* correction, int experts, int top,
                   int32_t* chosen, float* weights, int n, void* stream);
 int shk_moe_experts(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
-                    const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
-                    int dtype, int n, int width, int ff, int experts, int top, int act, void* stream);
+                    const void* w_up, const void* w_down, const void* add, const float* add_gate, int gate_ld,
+                    void* act_buf, void* out, int dtype, int n, int width, int ff, int experts, int top, int act, void* stream);
 // The same for bfloat16 on the matrix units, expert by expert over the lists of the (token,
 // expert) pairs that chose it (built on the device).  width and ff in multiples of 8; scratch:
 // shk_moe_grouped_scratch_bytes(...) bytes, 16-byte aligned.
 long long shk_moe_grouped_scratch_bytes(int n, int width, int experts, int top);
 int shk_moe_experts_grouped(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
-                            const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
-                            void* scratch, int n, int width, int ff, int experts, int top, int act, void* stream);
+                            const void* w_up, const void* w_down, const void* add, const float* add_gate,
+                            int gate_ld, void* act_buf, void* out, void* scratch, int n, int width, int ff, int experts, int top, int act, void* stream);
 
 // out = a_pos z^2 + z / 2 where z > 0, a_neg (exp(z) - 1 - z) + z / 2 elsewhere; elementwise.
 int shk_xielu(const void* x, void* out, int dtype, long long numel, float a_pos, float a_neg, void* stream);

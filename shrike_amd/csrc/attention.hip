@@ -9,7 +9,8 @@
 // operations: a token's result does not depend on how the step was cut.
 // Values may have another size than keys (v_dim); scores may be capped,
 // s <- cap * tanh(s / cap); and the softmax's denominator may hold one more
-// term per head, exp(sinks[head]), that has no key and no value.
+// term per head, exp(sinks[head]), that has no key and no value.  A learned bias by
+// distance, dist_bias[head][min(i - j, rows - 1)], may be added to the (capped) score.
 #include "api.h"
 #include "common.h"
 
@@ -27,7 +28,8 @@ __global__ void __launch_bounds__(kAttnThreads)
                              const int32_t* __restrict__ tables, int table_stride,
                              const T* __restrict__ k_pool, const T* __restrict__ v_pool,
                              int page_size, int num_pages, int window, int chunk, float scale,
-                             float softcap, const float* __restrict__ sinks) {
+                             float softcap, const float* __restrict__ sinks,
+                             const float* __restrict__ dist_bias, int bias_rows) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float probs[kAttnThreads];
   __shared__ int32_t rows[kAttnThreads];  // key-cache row of each key of the tile, -1 if masked
@@ -69,6 +71,8 @@ __global__ void __launch_bounds__(kAttnThreads)
         }
         s = dot * scale;
         if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        // a learned number per head and distance, the last row for every distance beyond the table
+        if (dist_bias) s += dist_bias[static_cast<size_t>(head) * bias_rows + min(pos - j, bias_rows - 1)];
       }
     }
     const float m_new = fmaxf(m_run, block_max(s, scratch));
@@ -122,8 +126,9 @@ extern "C" int shk_attention(const void* q, int q_stride, void* out, int dtype, 
                              const int32_t* token_seq, const int32_t* tables, int table_stride,
                              int num_seqs, const void* k_pool, const void* v_pool, int page_size,
                              int num_pages, int window, int chunk, float scale, int v_dim, float softcap,
-                             const float* sinks, void* stream) {
+                             const float* sinks, const float* dist_bias, int bias_rows, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "attention: unknown dtype %d", dtype);
+  SHK_REQUIRE(!dist_bias || bias_rows > 0, "attention: a distance bias needs a table of at least one row");
   SHK_REQUIRE(n >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
               "attention: heads=%d must be a positive multiple of kv_heads=%d", heads, kv_heads);
   SHK_REQUIRE(head_dim > 0 && head_dim <= kMaxHeadDim,
@@ -147,12 +152,14 @@ extern "C" int shk_attention(const void* q, int q_stride, void* out, int dtype, 
     attention_generic_kernel<float><<<grid, kAttnThreads, 0, s>>>(
         static_cast<const float*>(q), q_stride, static_cast<float*>(out), heads, kv_heads, head_dim, v_dim,
         positions, token_seq, tables, table_stride, static_cast<const float*>(k_pool),
-        static_cast<const float*>(v_pool), page_size, num_pages, window, chunk, scale, softcap, sinks);
+        static_cast<const float*>(v_pool), page_size, num_pages, window, chunk, scale, softcap, sinks, dist_bias,
+        bias_rows);
   else
     attention_generic_kernel<bf16><<<grid, kAttnThreads, 0, s>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, kv_heads, head_dim, v_dim,
         positions, token_seq, tables, table_stride, static_cast<const bf16*>(k_pool),
-        static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale, softcap, sinks);
+        static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale, softcap, sinks, dist_bias,
+        bias_rows);
   SHK_LAUNCH_CHECK("attention");
   return 0;
 }

@@ -94,6 +94,10 @@ const Launcher kLaunchers[] = {
     SHK_LAUNCHER(shk_moe_experts),
     SHK_LAUNCHER(shk_moe_experts_grouped),
     SHK_LAUNCHER(shk_embed_pairs),
+    SHK_LAUNCHER(shk_postnorm),
+    SHK_LAUNCHER(shk_cast_rows),
+    SHK_LAUNCHER(shk_activate),
+    SHK_LAUNCHER(shk_gate_mul),
     SHK_LAUNCHER(shk_argmax),
     SHK_LAUNCHER(shk_sample),
 };

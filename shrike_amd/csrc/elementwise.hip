@@ -148,16 +148,29 @@ __global__ void __launch_bounds__(kNormThreads)
 // ------------------------------------------------------------ act(gate) * up
 // act 1: SiLU, g / (1 + exp(-g)).  act 2: the tanh form of GELU,
 // 0.5 g (1 + tanh(u)), u = sqrt(2/pi) (g + 0.044715 g^3), written as g / (1 + exp(-2u)).
+// act 3: ReLU.  act 4: g sigmoid(1.702 g).  limit > 0 bounds the gate from above and the
+// other factor from both sides before anything else; up_shift is added to that factor.
 
 template <typename T>
-__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int act) {
+__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int act, float limit,
+                               float up_shift) {
   const size_t row = blockIdx.y;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= inter) return;
-  const float g = to_float(gu[row * 2 * inter + j]);
-  const float u = to_float(gu[row * 2 * inter + inter + j]);
-  const float x = act == 2 ? 2.f * 0.7978845608028654f * (g + 0.044715f * g * g * g) : g;
-  const float s = g / (1.f + expf(-x));
+  float g = to_float(gu[row * 2 * inter + j]);
+  float u = to_float(gu[row * 2 * inter + inter + j]);
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  u += up_shift;
+  float s;
+  if (act == 3) {
+    s = fmaxf(g, 0.f);
+  } else {
+    const float x = act == 2 ? 2.f * 0.7978845608028654f * (g + 0.044715f * g * g * g) : act == 4 ? 1.702f * g : g;
+    s = g / (1.f + expf(-x));
+  }
   out[row * inter + j] = from_float<T>(s * u);
 }
 
@@ -512,9 +525,11 @@ extern "C" int shk_add_rmsnorm(float* resid, const void* delta, const float* wei
   return 0;
 }
 
-extern "C" int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act, void* stream) {
+extern "C" int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act, float limit,
+                           float up_shift, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "act_mul: unknown dtype %d", dtype);
-  SHK_REQUIRE(act == 1 || act == 2, "act_mul: unknown activation %d", act);
+  SHK_REQUIRE(act >= 1 && act <= 4, "act_mul: unknown activation %d", act);
+  SHK_REQUIRE(limit >= 0.f, "act_mul: a limit must be positive (0: none), got %g", limit);
   SHK_REQUIRE(n >= 0 && inter > 0, "act_mul: bad sizes n=%d inter=%d", n, inter);
   if (n == 0) return 0;
   SHK_REQUIRE(n <= 65535, "act_mul: at most 65535 rows a call, got %d", n);
@@ -523,10 +538,10 @@ extern "C" int shk_act_mul(const void* gu, void* out, int dtype, int n, int inte
   dim3 grid((inter + 255) / 256, n);
   if (dtype == kF32)
     act_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gu),
-                                                static_cast<float*>(out), inter, act);
+                                                static_cast<float*>(out), inter, act, limit, up_shift);
   else
     act_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gu),
-                                               static_cast<bf16*>(out), inter, act);
+                                               static_cast<bf16*>(out), inter, act, limit, up_shift);
   SHK_LAUNCH_CHECK("act_mul");
   return 0;
 }

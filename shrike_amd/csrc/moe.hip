@@ -117,8 +117,15 @@ __global__ void __launch_bounds__(256)
 }
 
 __device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == 3) return fmaxf(g, 0.f);  // ReLU; with the gate's matrix also the other factor's, the square of ReLU
   const float x = act == 2 ? 2.f * 0.7978845608028654f * (g + 0.044715f * g * g * g) : g;
   return g / (1.f + expf(-x));
+}
+
+// What multiplies the shared expert's output for token t: sigmoid(add_gate[t * gate_ld]), one number
+// per token, or 1 without such a gate.
+__device__ __forceinline__ float shared_share(const float* __restrict__ add_gate, int gate_ld, int t) {
+  return add_gate ? 1.f / (1.f + expf(-add_gate[static_cast<size_t>(t) * gate_ld])) : 1.f;
 }
 
 constexpr int kMoeFeatures = 32;  // features (or columns) a workgroup
@@ -154,7 +161,8 @@ template <typename T>
 __global__ void __launch_bounds__(256)
     moe_down_kernel(const T* __restrict__ act_in, const int32_t* __restrict__ chosen,
                     const float* __restrict__ weights, const T* __restrict__ wd, const T* __restrict__ add,
-                    T* __restrict__ out, int width, int ff, int top, int experts) {
+                    const float* __restrict__ add_gate, int gate_ld, T* __restrict__ out, int width, int ff, int top,
+                    int experts) {
   extern __shared__ float as[];  // [top, ff]
   const int t = blockIdx.y;
   for (int i = threadIdx.x; i < top * ff; i += 256) as[i] = to_float(act_in[static_cast<size_t>(t) * top * ff + i]);
@@ -172,7 +180,7 @@ __global__ void __launch_bounds__(256)
       total = fmaf(weights[static_cast<size_t>(t) * top + k], wave_sum(d), total);
     }
     if (lane == 0) {
-      if (add) total += to_float(add[static_cast<size_t>(t) * width + c]);
+      if (add) total += shared_share(add_gate, gate_ld, t) * to_float(add[static_cast<size_t>(t) * width + c]);
       out[static_cast<size_t>(t) * width + c] = from_float<T>(total);
     }
   }
@@ -477,14 +485,14 @@ __global__ void __launch_bounds__(256)
 // out[t, c] = add[t, c] + sum_k weights[t, k] * pair_out[t * top + k, c], k in the order chosen
 __global__ void __launch_bounds__(256)
     moe_join_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, const bf16* __restrict__ add,
-                    bf16* __restrict__ out, int width, int top) {
+                    const float* __restrict__ add_gate, int gate_ld, bf16* __restrict__ out, int width, int top) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= width) return;
   float total = 0.f;
   for (int k = 0; k < top; ++k)
     total = fmaf(weights[static_cast<size_t>(t) * top + k], pair_out[(static_cast<size_t>(t) * top + k) * width + c], total);
-  if (add) total += to_float(add[static_cast<size_t>(t) * width + c]);
+  if (add) total += shared_share(add_gate, gate_ld, t) * to_float(add[static_cast<size_t>(t) * width + c]);
   out[static_cast<size_t>(t) * width + c] = from_float<bf16>(total);
 }
 
@@ -506,12 +514,13 @@ extern "C" int shk_moe_route(const float* logits, int ld, const float* correctio
 }
 
 extern "C" int shk_moe_experts(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
-                               const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
-                               int dtype, int n, int width, int ff, int experts, int top, int act, void* stream) {
+                               const void* w_up, const void* w_down, const void* add, const float* add_gate,
+                               int gate_ld, void* act_buf, void* out, int dtype, int n, int width, int ff, int experts, int top, int act, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_experts: unknown dtype %d", dtype);
   SHK_REQUIRE(n >= 0 && width > 0 && ff > 0 && experts > 0 && top >= 1 && top <= experts,
               "moe_experts: bad sizes n=%d width=%d ff=%d experts=%d top=%d", n, width, ff, experts, top);
-  SHK_REQUIRE(act == 1 || act == 2, "moe_experts: unknown activation %d", act);
+  SHK_REQUIRE(act >= 1 && act <= 3, "moe_experts: unknown activation %d", act);
+  SHK_REQUIRE(!add_gate || (add && gate_ld >= 1), "moe_experts: a gate of the added rows needs those rows and a stride");
   SHK_REQUIRE(width <= 15000 && static_cast<long long>(top) * ff <= 15000,
               "moe_experts: rows of %d, or %d chosen experts of %d features, do not fit a workgroup's LDS", width, top,
               ff);
@@ -527,7 +536,7 @@ extern "C" int shk_moe_experts(const void* x, const int32_t* chosen, const float
                                                                width, ff, top, act, experts);                         \
   moe_down_kernel<T><<<g2, 256, static_cast<size_t>(top) * ff * sizeof(float), s>>>(                                  \
       static_cast<const T*>(act_buf), chosen, weights, static_cast<const T*>(w_down), static_cast<const T*>(add),     \
-      static_cast<T*>(out), width, ff, top, experts)
+      add_gate, gate_ld, static_cast<T*>(out), width, ff, top, experts)
   if (dtype == kF32) {
     SHK_GO(float);
   } else {
@@ -545,12 +554,14 @@ extern "C" long long shk_moe_grouped_scratch_bytes(int n, int width, int experts
 }
 
 extern "C" int shk_moe_experts_grouped(const void* x, const int32_t* chosen, const float* weights, const void* w_gate,
-                                       const void* w_up, const void* w_down, const void* add, void* act_buf, void* out,
-                                       void* scratch, int n, int width, int ff, int experts, int top, int act,
+                                       const void* w_up, const void* w_down, const void* add, const float* add_gate,
+                                       int gate_ld, void* act_buf, void* out, void* scratch, int n, int width, int ff, int experts, int top, int act,
                                        void* stream) {
   SHK_REQUIRE(n >= 0 && width > 0 && ff > 0 && experts > 0 && experts <= 65535 && top >= 1 && top <= experts,
               "moe_experts_grouped: bad sizes n=%d width=%d ff=%d experts=%d top=%d", n, width, ff, experts, top);
-  SHK_REQUIRE(act == 1 || act == 2, "moe_experts_grouped: unknown activation %d", act);
+  SHK_REQUIRE(act >= 1 && act <= 3, "moe_experts_grouped: unknown activation %d", act);
+  SHK_REQUIRE(!add_gate || (add && gate_ld >= 1),
+              "moe_experts_grouped: a gate of the added rows needs those rows and a stride");
   SHK_REQUIRE(width % 8 == 0 && ff % 8 == 0, "moe_experts_grouped: width %d and ff %d must be multiples of 8", width, ff);
   if (n == 0) return 0;
   SHK_REQUIRE(static_cast<long long>(n) * top < (1LL << 30) && (n + 31) / 32 <= 65535,
@@ -582,8 +593,8 @@ extern "C" int shk_moe_experts_grouped(const void* x, const int32_t* chosen, con
     moe_down_mfma_kernel<<<dim3((width + 255) / 256, row_tiles, experts), 256, 0, s>>>(
         static_cast<const bf16*>(act_buf), order, counts, static_cast<const bf16*>(w_down), pair_out, n, width, ff, top);
   }
-  moe_join_kernel<<<dim3((width + 255) / 256, n), 256, 0, s>>>(pair_out, weights, static_cast<const bf16*>(add),
-                                                               static_cast<bf16*>(out), width, top);
+  moe_join_kernel<<<dim3((width + 255) / 256, n), 256, 0, s>>>(pair_out, weights, static_cast<const bf16*>(add), add_gate,
+                                                               gate_ld, static_cast<bf16*>(out), width, top);
   SHK_LAUNCH_CHECK("moe_experts_grouped");
   return 0;
 }

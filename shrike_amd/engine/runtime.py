@@ -40,22 +40,30 @@ class Runtime:
             return LinearWeight(w.shape, None, ops.retile_weight(w))
         return LinearWeight(w.shape, w, None)
 
-    def gated_weight(self, gate: torch.Tensor, up: torch.Tensor):
-        """The two matrices of a gated feed-forward, as `gated_linear` wants them."""
-        if self.dtype == torch.bfloat16:
+    @staticmethod
+    def fused_gate(activation: str = "silu", limit=None, up_shift: float = 0.0) -> bool:
+        """Whether the bfloat16 product's epilogue applies this gate itself."""
+        return activation in ("silu", "gelu_tanh") and limit is None and up_shift == 0.0
+
+    def gated_weight(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu", limit=None,
+                     up_shift: float = 0.0):
+        """The two matrices of a gated feed-forward, as `gated_linear` wants them for this gate."""
+        if self.dtype == torch.bfloat16 and self.fused_gate(activation, limit, up_shift):
             tiled = ops.interleave_gate_up(gate.contiguous(), up.contiguous())
             return LinearWeight(gate.shape, None, tiled)
         return self.weight(torch.cat([gate, up], dim=0))
 
-    def gated_linear(self, ctx, x, w: LinearWeight, out, activation: str = "silu") -> None:
-        """out = act(x @ gate.T) * (x @ up.T), act "silu" or "gelu_tanh".  bfloat16: one
-        product whose epilogue applies the activation; float32: product, then activation."""
-        if w.tiled is not None:
+    def gated_linear(self, ctx, x, w: LinearWeight, out, activation: str = "silu", limit=None,
+                     up_shift: float = 0.0) -> None:
+        """out = act(g) * (u + up_shift), g = x @ gate.T, u = x @ up.T, both bounded by `limit` first
+        where one is given.  bfloat16 with a gate that the product's epilogue applies: one product;
+        else product, then activation."""
+        if w.tiled is not None and self.fused_gate(activation, limit, up_shift):
             ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, gated=activation)
             return
         gate_up = ctx.buffer("ffn_gate_up", (x.shape[0], w.rows), self.dtype)
-        ops.gemm(x, w.dense, gate_up)
-        ops.act_mul(gate_up, out, activation)
+        self.linear(x, w, gate_up)
+        ops.act_mul(gate_up, out, activation, limit, up_shift)
 
     def linear(self, x, w: LinearWeight, out, bias=None, accumulate=False) -> None:
         """out (+)= x @ w.T + bias."""

@@ -34,7 +34,11 @@ _SIGNATURES = {
     "shk_add_normed_rmsnorm": [_P, _P, _I, _P, _F, _P, _F, _P, _I, _P, _I, _I, _I, _I, _P],
     "shk_act_mul_rows": [_P, _I, _P, _I, _P, c_longlong, _I, _I, _P, _I, _I, _I, _P],
     "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _I, _I, _P],
-    "shk_act_mul": [_P, _P, _I, _I, _I, _I, _P],
+    "shk_act_mul": [_P, _P, _I, _I, _I, _I, _F, _F, _P],
+    "shk_postnorm": [_P, _P, _I, _F, _P, _P, _F, _P, _I, _I, _I, _P],
+    "shk_cast_rows": [_P, _P, _I, c_longlong, _P],
+    "shk_activate": [_P, _P, _I, c_longlong, _I, _P],
+    "shk_gate_mul": [_P, _P, _P, _I, c_longlong, _P],
     "shk_gemm": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "shk_retile_weight": [_P, _I, _I, _P, _P],
     "shk_interleave_gate_up": [_P, _P, _I, _I, _P, _P],
@@ -44,8 +48,9 @@ _SIGNATURES = {
     "shk_mfma_alone": [_P, _P, _I, _I, _P],
     "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _I, _I,
                           _P],
-    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _P, _P],
-    "shk_qkv_store": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _P, _P,
+                      _I, _P],
+    "shk_qkv_store": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
     "shk_latent_prepare": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
     "shk_rotate_heads": [_P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P],
     "shk_latent_attention": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
@@ -68,8 +73,8 @@ _SIGNATURES = {
     "shk_rotate_half_rows": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _I, _P],
     "shk_retention_scan": [_P, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, c_longlong, _P, _P],
     "shk_moe_route": [_P, _I, _P, _I, _I, _P, _P, _I, _P],
-    "shk_moe_experts": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-    "shk_moe_experts_grouped": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "shk_moe_experts": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "shk_moe_experts_grouped": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_xielu": [_P, _P, _I, c_longlong, _F, _F, _P],
     "shk_embed_pairs": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],

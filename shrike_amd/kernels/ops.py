@@ -241,7 +241,11 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_resid=Tr
     )
 
 
-GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}
+# a gate's activation: SiLU, GELU in its tanh form, ReLU, g * sigmoid(1.702 g); the products with a fused
+# activation, the experts' kernels and act_mul each say which of them they take
+GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2, "relu": 3, "quick_gelu": 4}
+# an activation of a plain product (activate): the above without a second factor, and the square of ReLU
+PLAIN_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2, "relu": 3, "relu_squared": 4}
 
 
 def activation_code(gated) -> int:
@@ -256,15 +260,63 @@ def activation_code(gated) -> int:
         raise KernelError(f"gate activation must be one of {sorted(GATE_ACTIVATIONS)}, got {gated!r}") from None
 
 
-def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
-    """out = act(gate_up[:, :I]) * gate_up[:, I:]."""
+def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu", limit: float | None = None,
+            up_shift: float = 0.0) -> None:
+    """out = act(g) * (u + up_shift) with g = gate_up[:, :I], u = gate_up[:, I:]; with `limit`,
+    g <- min(g, limit) and u <- clamp(u, -limit, limit) first."""
     n, inter = out.shape
     if gate_up.shape != (n, 2 * inter) or not gate_up.is_contiguous() or not out.is_contiguous():
         raise KernelError("act_mul: gate_up must be contiguous [n, 2*inter]")
     if gate_up.dtype != out.dtype:
         raise KernelError("act_mul: dtypes differ")
     check(load().shk_act_mul(_dev(gate_up, "gate_up"), _dev(out, "out"), dtype_code(out.dtype),
-                             n, inter, activation_code(activation), _stream()))
+                             n, inter, activation_code(activation), float(limit or 0.0), float(up_shift), _stream()))
+
+
+def postnorm(resid, delta, alpha: float, lscale, weight, eps: float, cast=None, dtype=None) -> None:
+    """resid <- rmsnorm(alpha * resid + lscale * delta) * weight, row by row in float32 (lscale float32
+    [hidden] or None: ones; delta a tensor of the compute dtype or a SplitSum); `cast`, if given,
+    receives the new rows in the compute dtype."""
+    n, hidden = resid.shape
+    dtype = cast.dtype if cast is not None else dtype
+    if dtype is None:
+        raise KernelError("postnorm: give cast or dtype")
+    if not resid.is_contiguous() or (cast is not None and (cast.shape != resid.shape or not cast.is_contiguous())):
+        raise KernelError("postnorm: resid and cast must be contiguous and of one shape")
+    if weight.numel() != hidden or (lscale is not None and lscale.numel() != hidden):
+        raise KernelError(f"postnorm: weight and lscale must have {hidden} elements")
+    p, splits = _delta(delta, resid, dtype, "postnorm")
+    check(load().shk_postnorm(_dev(resid, "resid", torch.float32), p, splits, float(alpha),
+                              None if lscale is None else _dev(lscale, "lscale", torch.float32),
+                              _dev(weight, "weight", torch.float32), float(eps),
+                              None if cast is None else _dev(cast, "cast"), dtype_code(dtype), n, hidden, _stream()))
+
+
+def cast_rows(src, dst) -> None:
+    """dst = src (float32) in dst's dtype."""
+    if src.shape != dst.shape or not src.is_contiguous() or not dst.is_contiguous():
+        raise KernelError("cast_rows: src and dst must be contiguous and of one shape")
+    check(load().shk_cast_rows(_dev(src, "src", torch.float32), _dev(dst, "dst"), dtype_code(dst.dtype), src.numel(),
+                               _stream()))
+
+
+def activate(x, out, activation: str) -> None:
+    """out = act(x) elementwise, act one of PLAIN_ACTIVATIONS."""
+    if x.shape != out.shape or x.dtype != out.dtype or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError("activate: x and out must be contiguous and alike")
+    if activation not in PLAIN_ACTIVATIONS:
+        raise KernelError(f"activate: activation must be one of {sorted(PLAIN_ACTIVATIONS)}, got {activation!r}")
+    check(load().shk_activate(_dev(x, "x"), _dev(out, "out"), dtype_code(x.dtype), x.numel(),
+                              PLAIN_ACTIVATIONS[activation], _stream()))
+
+
+def gate_mul(x, gate, out) -> None:
+    """out = x * sigmoid(gate) elementwise."""
+    if x.shape != out.shape or gate.shape != x.shape or x.dtype != out.dtype or gate.dtype != x.dtype \
+            or not (x.is_contiguous() and gate.is_contiguous() and out.is_contiguous()):
+        raise KernelError("gate_mul: x, gate and out must be contiguous and alike")
+    check(load().shk_gate_mul(_dev(x, "x"), _dev(gate, "gate"), _dev(out, "out"), dtype_code(x.dtype), x.numel(),
+                              _stream()))
 
 
 def gemm(a, w, out, bias=None, accumulate=False) -> None:
@@ -451,10 +503,11 @@ def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, 
 
 
 def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k_pool, v_pool,
-              page_size, window, scale, chunk=None, v_dim=None, softcap=None, sinks=None) -> None:
+              page_size, window, scale, chunk=None, v_dim=None, softcap=None, sinks=None, dist_bias=None) -> None:
     """q: [n, >= heads*head_dim] rows (a view into qkv is fine); out [n, heads*v_dim].
     v_dim: size of a value (None: head_dim); softcap: scores become cap * tanh(score / cap);
-    sinks: float32 [heads], one more term exp(sinks[h]) in each head's softmax denominator."""
+    sinks: float32 [heads], one more term exp(sinks[h]) in each head's softmax denominator;
+    dist_bias: float32 [heads, rows], dist_bias[h, min(i - j, rows - 1)] joins the (capped) score."""
     _rows(q, "attention q")
     n = q.shape[0]
     v_dim = head_dim if v_dim is None else int(v_dim)
@@ -462,6 +515,7 @@ def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k
         raise KernelError("attention: out must be contiguous [n, heads*v_dim] of q's dtype")
     if sinks is not None and (sinks.numel() != heads or not sinks.is_contiguous()):
         raise KernelError(f"attention: sinks must hold one value per head ({heads})")
+    _dist_bias(dist_bias, heads, "attention")
     _check_pools("attention", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size, v_dim)
     check(
         load().shk_attention(
@@ -470,20 +524,39 @@ def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k
             _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], tables.shape[0], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"),
             page_size, k_pool.shape[0], int(window or 0), int(chunk or 0), float(scale), v_dim,
-            float(softcap or 0.0), None if sinks is None else _dev(sinks, "sinks", torch.float32), _stream(),
+            float(softcap or 0.0), None if sinks is None else _dev(sinks, "sinks", torch.float32),
+            None if dist_bias is None else _dev(dist_bias, "dist_bias", torch.float32),
+            0 if dist_bias is None else dist_bias.shape[1], _stream(),
         )
     )
 
 
+def _dist_bias(dist_bias, heads, who):
+    if dist_bias is not None and (dist_bias.dim() != 2 or dist_bias.shape[0] != heads or dist_bias.shape[1] < 1
+                                  or not dist_bias.is_contiguous() or dist_bias.dtype != torch.float32):
+        raise KernelError(f"{who}: a distance bias must be contiguous float32 [heads ({heads}), rows]")
+
+
 def qkv_store(qkv, heads, kv_heads, head_dim, v_dim, positions, token_seq, tables, k_pool, v_pool, page_size,
-              q_temperature=None, v_norm_eps=None, write_kv=True) -> None:
+              q_temperature=None, v_norm_eps=None, write_kv=True, qk_norm_eps=None, q_weight=None, k_weight=None,
+              has_kv=True) -> None:
     """Cache write without rotation for keys of head_dim and values of v_dim: qkv is [n, heads *
     head_dim + kv_heads * (head_dim + v_dim)].  q_temperature = (coef, every): the queries at
     position p are multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) in place.
-    v_norm_eps: each head's value is stored divided by sqrt(mean(v^2) + eps)."""
+    v_norm_eps: each head's value is stored divided by sqrt(mean(v^2) + eps).
+    qk_norm_eps: every head of the queries (in place, before the temperature) and of the keys is
+    divided by sqrt(mean(x^2) + eps) and multiplied by q_weight / k_weight (float32 [head_dim], or
+    None).  has_kv False: qkv is [n, heads * head_dim], queries alone; nothing is written."""
     n = qkv.shape[0]
-    if not qkv.is_contiguous() or qkv.shape[1] != heads * head_dim + kv_heads * (head_dim + v_dim):
-        raise KernelError("qkv_store: qkv must be contiguous [n, heads*head_dim + kv_heads*(head_dim + v_dim)]")
+    write_kv = bool(write_kv and has_kv)
+    width = heads * head_dim + (kv_heads * (head_dim + v_dim) if has_kv else 0)
+    if not qkv.is_contiguous() or qkv.shape[1] != width:
+        raise KernelError("qkv_store: qkv must be contiguous [n, heads*head_dim + kv_heads*(head_dim + v_dim)] "
+                          "(queries alone without has_kv)")
+    for w in (q_weight, k_weight):
+        if w is not None and (qk_norm_eps is None or w.numel() != head_dim or w.dtype != torch.float32
+                              or not w.is_contiguous()):
+            raise KernelError("qkv_store: norm weights are float32 [head_dim] and need qk_norm_eps")
     if positions.shape[0] < n or (write_kv and token_seq.shape[0] < n):
         raise KernelError(f"qkv_store: qkv has {n} rows but positions / token_seq are shorter")
     num_pages = 0
@@ -495,7 +568,9 @@ def qkv_store(qkv, heads, kv_heads, head_dim, v_dim, positions, token_seq, table
         raise KernelError(f"qkv_store: the query temperature's step must be positive, got {every}")
     check(load().shk_qkv_store(
         _dev(qkv, "qkv"), dtype_code(qkv.dtype), n, heads, kv_heads, head_dim, v_dim, coef, every,
-        float(v_norm_eps or 0.0), _dev(positions, "positions", torch.int32),
+        float(v_norm_eps or 0.0), float(qk_norm_eps or 0.0),
+        None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
+        int(bool(has_kv)), _dev(positions, "positions", torch.int32),
         _dev(token_seq, "token_seq", torch.int32) if write_kv else None,
         _dev(tables, "tables", torch.int32) if write_kv else None, tables.shape[1] if write_kv else 0,
         _dev(k_pool, "k_pool") if write_kv else None, _dev(v_pool, "v_pool") if write_kv else None,
@@ -952,10 +1027,13 @@ def moe_grouped_scratch_bytes(n: int, width: int, experts: int, top: int) -> int
 
 
 def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activation: str = "silu", add=None,
-                scratch=None) -> None:
+                scratch=None, add_gate=None) -> None:
     """out = add + sum_k weights[:, k] * down_e(act(gate_e x) * up_e x), e = chosen[:, k]; matrices
     stacked [experts, ff, width] / [experts, width, ff] row-major in x's dtype.  scratch (uint8,
-    moe_grouped_scratch_bytes): the products run per expert on the matrix units (see moe_grouped)."""
+    moe_grouped_scratch_bytes): the products run per expert on the matrix units (see moe_grouped).
+    add_gate: a float32 column (a view [n] with any stride): add[t] is multiplied by
+    sigmoid(add_gate[t]).  Experts without a gate whose activation is the square of ReLU pass
+    their one matrix as both w_gate and w_up with activation "relu"."""
     n, width = x.shape
     experts, ff, _ = w_gate.shape
     top = chosen.shape[1]
@@ -967,6 +1045,11 @@ def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activati
             or act_buf.numel() < n * top * ff or (add is not None and tuple(add.shape) != (n, width)) \
             or tuple(weights.shape) != (n, top) or chosen.dtype != torch.int32 or weights.dtype != torch.float32:
         raise KernelError("moe_experts: mismatched shapes")
+    gate_ptr, gate_ld = None, 0
+    if add_gate is not None:
+        if add is None or add_gate.dtype != torch.float32 or add_gate.dim() != 1 or add_gate.shape[0] != n:
+            raise KernelError("moe_experts: add_gate is a float32 column of n numbers and needs `add`")
+        gate_ptr, gate_ld = _dev(add_gate, "add_gate"), max(1, add_gate.stride(0))
     if scratch is not None:
         if not moe_grouped(n, width, ff, x.dtype) or scratch.dtype != torch.uint8 \
                 or scratch.numel() < moe_grouped_scratch_bytes(n, width, experts, top):
@@ -974,13 +1057,13 @@ def moe_experts(x, chosen, weights, w_gate, w_up, w_down, act_buf, out, activati
                               "moe_grouped_scratch_bytes() bytes")
         check(load().shk_moe_experts_grouped(
             _dev(x, "x"), _dev(chosen, "chosen"), _dev(weights, "weights"), _dev(w_gate, "w_gate"), _dev(w_up, "w_up"),
-            _dev(w_down, "w_down"), None if add is None else _dev(add, "add"), _dev(act_buf, "act_buf"),
-            _dev(out, "out"), _dev(scratch, "scratch"), n, width, ff, experts, top, activation_code(activation),
+            _dev(w_down, "w_down"), None if add is None else _dev(add, "add"), gate_ptr, gate_ld,
+            _dev(act_buf, "act_buf"), _dev(out, "out"), _dev(scratch, "scratch"), n, width, ff, experts, top, activation_code(activation),
             _stream()))
         return
     check(load().shk_moe_experts(_dev(x, "x"), _dev(chosen, "chosen"), _dev(weights, "weights"), _dev(w_gate, "w_gate"),
                                  _dev(w_up, "w_up"), _dev(w_down, "w_down"), None if add is None else _dev(add, "add"),
-                                 _dev(act_buf, "act_buf"), _dev(out, "out"), dtype_code(x.dtype), n, width, ff, experts,
+                                 gate_ptr, gate_ld, _dev(act_buf, "act_buf"), _dev(out, "out"), dtype_code(x.dtype), n, width, ff, experts,
                                  top, activation_code(activation), _stream()))
 
 

@@ -147,6 +147,7 @@ class DecoderModel:
                 if entry.add_vector is not None:
                     vector = self.stream_vectors[entry.add_vector[0]][entry.add_vector[1]]
                 ops.add_rows(hidden.resid, embedded if entry.add_embedding else None, vector)
+                hidden.cast = None
             self.blocks[entry.block].forward(ctx, hidden, caches[pos])
             if history is not None:
                 # the run's result is its stream plus what is pending; a pending output with a

@@ -49,6 +49,25 @@ def kv_cache_spec(num_kv_heads: int, head_dim: int, window: int | None = None,
     )
 
 
+def distance_buckets(rows: int, reach: int) -> list[int]:
+    """Row of a [rows, heads] bias table for every distance 0 .. reach between a query and a key:
+    with half = rows // 2, the distances below half have a row each; from there on the row is half
+    + floor(ln(d / half) / ln(reach / half) * (rows - half)), the rest of the rows spread evenly over
+    the logarithm of the distance up to `reach`; the last row serves that distance and all beyond."""
+    import math
+
+    half = rows // 2
+    out = []
+    for d in range(reach + 1):
+        if d < half:
+            out.append(d)
+        elif half <= 0 or reach <= half:
+            out.append(rows - 1)
+        else:
+            out.append(min(rows - 1, half + math.floor(math.log(d / half) / math.log(reach / half) * (rows - half))))
+    return out
+
+
 def _pow2(n: int, floor: int = 1) -> int:
     b = floor
     while b < n:
@@ -168,7 +187,13 @@ class PagedAttention(Mixer):
         s = self.spec
         return bool(self.value_dim != s.head_dim or getattr(s, "query_temperature", None)
                     or getattr(s, "value_norm_eps", None) or getattr(s, "softcap", None)
-                    or getattr(s, "sinks", False) or self.talking)
+                    or getattr(s, "sinks", False) or self.talking or getattr(s, "qk_norm", None)
+                    or getattr(s, "bucket_bias", None) or self.shared_kv)
+
+    @property
+    def shared_kv(self) -> bool:
+        """Whether the layer has no keys and values of its own and reads another run's cache."""
+        return bool(getattr(self.spec, "shared_kv", False))
 
     @property
     def talking(self) -> bool:
@@ -182,10 +207,22 @@ class PagedAttention(Mixer):
         s, h = self.spec, self.width
         q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
         t = self._tensor
-        out = [ParamSpec(t("q"), (q, h)), ParamSpec(t("k"), (kv, h))]
-        if not s.values_from_keys:
-            out.append(ParamSpec(t("v"), (s.num_kv_heads * self.value_dim, h)))
+        out = [ParamSpec(t("q"), (q, h))]
+        if not self.shared_kv:
+            out.append(ParamSpec(t("k"), (kv, h)))
+            if not s.values_from_keys:
+                out.append(ParamSpec(t("v"), (s.num_kv_heads * self.value_dim, h)))
         out.append(ParamSpec(t("o"), (h, s.num_heads * self.value_dim)))
+        qk_norm = getattr(s, "qk_norm", None)
+        if qk_norm and qk_norm[1]:
+            out.append(ParamSpec(t("q_norm"), (s.head_dim,), init="norm", keep_float32=True))
+            if not self.shared_kv:
+                out.append(ParamSpec(t("k_norm"), (s.head_dim,), init="norm", keep_float32=True))
+        if getattr(s, "bucket_bias", None):
+            # (rows None: the table has as many rows as the file's tensor; random weights then draw 32)
+            rows = s.bucket_bias[0]
+            out.append(ParamSpec(t("rel"), (None if rows is None else int(rows), s.num_heads), init="bias",
+                                 keep_float32=True, free_size=32))
         if getattr(s, "sinks", False):
             out.append(ParamSpec(t("sink"), (s.num_heads,), init="bias", keep_float32=True))
         if getattr(s, "distance_bias", False):
@@ -202,14 +239,16 @@ class PagedAttention(Mixer):
 
     _DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-                      "o_bias": "o_proj.bias", "sink": "sinks", "r1": "r1", "r2": "r2", "talk": "talk"}
+                      "o_bias": "o_proj.bias", "sink": "sinks", "r1": "r1", "r2": "r2", "talk": "talk",
+                      "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "rel": "rel"}
 
     def _tensor(self, role: str) -> str:
         return self.tensor_name(role, self._DEFAULT_NAMES[role])
 
     def cache_spec(self):
         s = self.spec
-        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window, s.chunk,
+        kept = getattr(s, "cache_window", "own")
+        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window if kept == "own" else kept, s.chunk,
                              None if self.value_dim == s.head_dim else self.value_dim)
 
     def check(self, runtime):
@@ -226,6 +265,18 @@ class PagedAttention(Mixer):
                 raise ValueError(f"{self.name}: query_temperature must be (coef, every) with every >= 1, got {qt}")
             if getattr(s, "softcap", None) is not None and not s.softcap > 0:
                 raise ValueError(f"{self.name}: softcap must be positive, got {s.softcap}")
+        qk_norm, buckets = getattr(s, "qk_norm", None), getattr(s, "bucket_bias", None)
+        if qk_norm is not None and (len(qk_norm) != 2 or not float(qk_norm[0]) > 0):
+            raise ValueError(f"{self.name}: qk_norm must be (eps > 0, weighted), got {qk_norm}")
+        if buckets is not None and (len(buckets) != 2 or (buckets[0] is not None and int(buckets[0]) < 1)
+                                    or int(buckets[1]) < 1):
+            raise ValueError(f"{self.name}: bucket_bias must be (rows >= 1, reach >= 1), got {buckets}")
+        if self.talking and (qk_norm or buckets or self.shared_kv):
+            raise ValueError(f"{self.name}: a distance bias by formula, a fixed sink and mixed heads are built "
+                             "without normed queries and keys, a bias table and a cache of another layer")
+        kept = getattr(s, "cache_window", "own")
+        if kept != "own" and kept is not None and (s.window is None or kept < s.window):
+            raise ValueError(f"{self.name}: the cache keeps {kept} keys, fewer than the layer's own window")
         if self.talking and (getattr(s, "sinks", False) or getattr(s, "softcap", None)
                              or getattr(s, "query_temperature", None) or getattr(s, "value_norm_eps", None)):
             raise ValueError(f"{self.name}: a distance bias, a fixed sink and mixed heads are built without "
@@ -248,7 +299,7 @@ class PagedAttention(Mixer):
 
     def load(self, tensors, runtime):
         s, t = self.spec, self._tensor
-        roles = ("q", "k") if s.values_from_keys else ("q", "k", "v")
+        roles = ("q",) if self.shared_kv else ("q", "k") if s.values_from_keys else ("q", "k", "v")
         self.w_qkv = runtime.weight(torch.cat([tensors[t(r)] for r in roles], dim=0))
         self.b_qkv = torch.cat([tensors[t(f"{r}_bias")] for r in roles]).contiguous() if s.qkv_bias else None
         self.w_o = runtime.weight(tensors[t("o")])
@@ -258,6 +309,17 @@ class PagedAttention(Mixer):
         self.r1 = tensors[t("r1")].contiguous() if bias else None
         self.r2 = tensors[t("r2")].contiguous() if bias else None
         self.talk = tensors[t("talk")].contiguous() if getattr(s, "talking_heads", False) else None
+        qk_norm = getattr(s, "qk_norm", None)
+        self.q_norm = self.k_norm = None
+        if qk_norm and qk_norm[1]:
+            self.q_norm = tensors[t("q_norm")].contiguous()
+            self.k_norm = None if self.shared_kv else tensors[t("k_norm")].contiguous()
+        self.dist_bias = None
+        if getattr(s, "bucket_bias", None):
+            # the table by distance, a row per head: the kernels look a distance up, not its bucket
+            rows, reach = int(tensors[t("rel")].shape[0]), int(s.bucket_bias[1])
+            index = torch.tensor(distance_buckets(rows, reach), dtype=torch.long, device=tensors[t("rel")].device)
+            self.dist_bias = tensors[t("rel")].to(torch.float32)[index].t().contiguous()
         if self.position is not None:
             self.position.load(tensors, runtime)
         self.linear = runtime.linear
@@ -270,7 +332,8 @@ class PagedAttention(Mixer):
     def plan_key(self):
         s = self.spec
         return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window, s.chunk, self.plain_store,
-                self.talking)
+                self.talking, self.value_dim, self._qkv_width(), bool(getattr(s, "bucket_bias", None)),
+                bool(getattr(s, "softcap", None)), bool(getattr(s, "sinks", False)))
 
     def prepare(self, shape) -> None:
         """Decides once per step and head geometry how attention is launched:
@@ -317,6 +380,8 @@ class PagedAttention(Mixer):
             return
         plan.mfma = self.dtype == torch.bfloat16 and self.value_dim == d and ops.attention_supports_mfma(
             h, hkv, d, shape.page_size, self._qkv_width())
+        if getattr(s, "bucket_bias", None):
+            plan.mfma = False
         # capped scores and sinks are built into the decode kernel and the shared-key prompt
         # kernel; where the latter does not take the shape, the general kernel serves the step
         if plan.mfma and (getattr(s, "softcap", None) or getattr(s, "sinks", False)) \
@@ -399,7 +464,8 @@ class PagedAttention(Mixer):
         if not plan.mfma:
             ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.pools["k"],
                           cache.pools["v"], cache.page_size, s.window, s.scale, chunk=s.chunk,
-                          v_dim=self.value_dim, softcap=getattr(s, "softcap", None), sinks=self.sinks)
+                          v_dim=self.value_dim, softcap=getattr(s, "softcap", None), sinks=self.sinks,
+                          dist_bias=self.dist_bias)
             return
         if ctx.num_decode:
             partial = ctx.buffer("attn_partial", (ctx.num_decode * h * plan.nsplit * (d + 2),),
@@ -428,6 +494,8 @@ class PagedAttention(Mixer):
 
     def _qkv_width(self) -> int:
         s = self.spec
+        if self.shared_kv:
+            return s.num_heads * s.head_dim
         if s.values_from_keys:
             return (s.num_heads + s.num_kv_heads) * s.head_dim
         return (s.num_heads + s.num_kv_heads) * s.head_dim + s.num_kv_heads * self.value_dim
@@ -437,13 +505,19 @@ class PagedAttention(Mixer):
         n = x.shape[0]
         qkv_width = self._qkv_width()
         if self.plain_store:
+            qk_norm = getattr(s, "qk_norm", None)
+            if self.shared_kv == cache.owned:
+                raise RuntimeError(f"{self.name}: a layer without keys and values of its own must read another "
+                                   "run's cache, and only such a layer may")
             qkv = ctx.buffer("attn_qkv", (n, qkv_width), ctx.dtype)
             self.linear(x, self.w_qkv, qkv)
             tables = ctx.block_tables[cache.group]
             ops.qkv_store(qkv, s.num_heads, s.num_kv_heads, s.head_dim, self.value_dim, ctx.positions,
                           ctx.token_seq, tables, cache.pools["k"], cache.pools["v"], cache.page_size,
                           q_temperature=getattr(s, "query_temperature", None),
-                          v_norm_eps=getattr(s, "value_norm_eps", None), write_kv=cache.owned)
+                          v_norm_eps=getattr(s, "value_norm_eps", None), write_kv=cache.owned,
+                          qk_norm_eps=qk_norm[0] if qk_norm else None, q_weight=self.q_norm, k_weight=self.k_norm,
+                          has_kv=not self.shared_kv)
             attn = ctx.buffer("attn_out", (n, s.num_heads * self.value_dim), ctx.dtype)
             self.attend(ctx, qkv, attn, tables, cache)
             return self.linear_deferred(ctx, "attn_proj", attn, self.w_o, bias=self.b_o)

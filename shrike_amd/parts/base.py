@@ -45,13 +45,27 @@ class ParamSpec:
         a "matrix" by its fan-in and leaves an "embedding" at N(0, 1).
     keep_float32: held in float32 whatever the compute dtype (vectors that
         enter float32 arithmetic); others are held in the compute dtype.
+    shape: a size may be None where the file's tensor decides it (the rows of a
+        table that config.json does not count); random weights then take
+        `free_size` for it.
     """
 
     name: str
-    shape: tuple[int, ...]
+    shape: tuple
     init: str = "matrix"
     keep_float32: bool = False
     optional: bool = False
+    free_size: int = 1
+
+    def matches(self, shape) -> bool:
+        """Whether a file's tensor of this shape is what the part declared."""
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(
+            (want is None and got >= 1) or want == got for want, got in zip(self.shape, shape))
+
+    def drawn_shape(self) -> tuple[int, ...]:
+        """The shape that random weights take."""
+        return tuple(self.free_size if d is None else int(d) for d in self.shape)
 
 
 PAGE = "page"  # in a PageTensor's dims: the place of the page size
@@ -142,14 +156,16 @@ class HiddenState:
     `pending_norm` = (weight float32 [width], eps) says that `pending` joins the
     stream as pending * rsqrt(mean(pending^2) + eps) * weight, row by row;
     (weight, bias, eps) that it joins as its layer norm, (pending - mean) /
-    sqrt(var + eps) * weight + bias."""
+    sqrt(var + eps) * weight + bias.  `cast`: the stream as it stands (nothing pending) in the
+    compute dtype, where the kernel that wrote `resid` last left such a copy."""
 
-    __slots__ = ("resid", "pending", "pending_norm")
+    __slots__ = ("resid", "pending", "pending_norm", "cast")
 
     def __init__(self, resid: torch.Tensor, pending: torch.Tensor | None = None, pending_norm=None):
         self.resid = resid
         self.pending = pending
         self.pending_norm = pending_norm
+        self.cast = None
 
     def settle(self, ctx) -> None:
         """Adds what is pending to `resid` now (for a reader that is no norm)."""
@@ -157,6 +173,7 @@ class HiddenState:
 
         if self.pending is None:
             return
+        self.cast = None
         if self.pending_norm is not None and len(self.pending_norm) == 3:
             ops.add_layernorm(self.resid, self.pending, dnorm=self.pending_norm, dtype=ctx.dtype)
         elif self.pending_norm is not None:

@@ -160,3 +160,87 @@ class SandwichResidualBlock(Block):
 
 
 register_block("sandwich_residual", SandwichResidualBlock)
+
+
+class PostNormResidualBlock(Block):
+    """x <- norm1(alpha x + s1 * mixer(x)); x <- norm2(alpha x + s2 * ffn(x)): the norm stands
+    after the sum, the stream is what the norm leaves, and the sublayers read the stream itself.
+    One kernel per sublayer forms the scaled sum in float32 (adding up the parts of a split
+    product in order), norms it, stores it as the float32 stream and leaves it in the compute
+    dtype for the products that read it next."""
+
+    def __init__(self, spec, width, name):
+        super().__init__(spec, width, name)
+        self.mixer = build_part("mixer", spec.mixer, width, f"{name}.{spec.mixer_name}")
+        self.mixer_norm = build_part("norm", spec.mixer_norm, width, f"{name}.{spec.mixer_norm_name}")
+        self.ffn = self.ffn_norm = None
+        if spec.ffn is not None:
+            self.ffn = build_part("ffn", spec.ffn, width, f"{name}.{spec.ffn_name}")
+            self.ffn_norm = build_part("norm", spec.ffn_norm, width, f"{name}.{spec.ffn_norm_name}")
+        self.parts = tuple(p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None)
+        self.parts += tuple(getattr(self.mixer, "parts", ()))
+        self.mixer_scale = self.ffn_scale = None
+
+    def _own(self):
+        return tuple(p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None)
+
+    def _scale_names(self):
+        s = self.spec
+        if not s.layer_scale:
+            return ()
+        return (f"{self.name}.{s.mixer_scale_name}",) + ((f"{self.name}.{s.ffn_scale_name}",) if self.ffn else ())
+
+    def params(self):
+        from .base import ParamSpec
+
+        out = [p for part in self._own() for p in part.params()]
+        return out + [ParamSpec(n, (self.width,), init="norm", keep_float32=True) for n in self._scale_names()]
+
+    def check(self, runtime):
+        for part in (self.mixer_norm, self.ffn_norm):
+            if part is not None and (getattr(part.spec, "kind", None) != "rmsnorm"):
+                raise ValueError(f"{self.name}: the norm after a sum must be an RMS norm (rmsnorm)")
+        for part in self._own():
+            part.check(runtime)
+
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for part in self.parts)
+
+    @property
+    def launches_follow_shape(self):
+        return all(part.launches_follow_shape for part in self.parts)
+
+    def load(self, tensors, runtime):
+        for part in self._own():
+            part.load(tensors, runtime)
+        names = self._scale_names()
+        if names:
+            self.mixer_scale = tensors[names[0]].contiguous()
+            self.ffn_scale = tensors[names[1]].contiguous() if self.ffn else None
+        self.alpha = float(self.spec.alpha)
+
+    def forward(self, ctx, hidden: HiddenState, cache) -> None:
+        import torch
+
+        from ..kernels import ops
+
+        hidden.settle(ctx)
+        in_float32 = ctx.dtype == torch.float32
+        x = hidden.resid if in_float32 else hidden.cast
+        if x is None:
+            x = ctx.buffer("stream_cast", hidden.resid.shape, ctx.dtype)
+            ops.cast_rows(hidden.resid, x)
+        out = None if in_float32 else ctx.buffer("stream_cast", hidden.resid.shape, ctx.dtype)
+        mixed = self.mixer.forward(ctx, x, cache)
+        ops.postnorm(hidden.resid, mixed, self.alpha, self.mixer_scale, self.mixer_norm.weight, self.mixer_norm.eps,
+                     cast=out, dtype=ctx.dtype)
+        if self.ffn is not None:
+            x = hidden.resid if in_float32 else out
+            fed = self.ffn.forward(ctx, x)
+            ops.postnorm(hidden.resid, fed, self.alpha, self.ffn_scale, self.ffn_norm.weight, self.ffn_norm.eps,
+                         cast=out, dtype=ctx.dtype)
+        hidden.cast = out
+
+
+register_block("postnorm_residual", PostNormResidualBlock)

@@ -31,7 +31,8 @@ class LatentAttention(Mixer):
         y = W_o o                                     product
 
     and the attention itself is that of one shared key/value head of size kv_rank +
-    rot_dim: what is read per cached token does not grow with the number of heads."""
+    rot_dim: what is read per cached token does not grow with the number of heads.  With the
+    spec's output gate, o is multiplied by sigmoid(W_g x) before the last product."""
 
     launches_follow_shape = True
 
@@ -41,7 +42,8 @@ class LatentAttention(Mixer):
     def params(self):
         s, h = self.spec, self.width
         H = s.num_heads
-        return [
+        gate = [ParamSpec(self._t("g"), (H * s.value_dim, h))] if getattr(s, "output_gate", False) else []
+        return gate + [
             ParamSpec(self._t("dq"), (s.q_rank, h)),
             ParamSpec(self._t("dq.norm"), (s.q_rank,), init="norm", keep_float32=True),
             ParamSpec(self._t("uq"), (H * (s.head_dim + s.rot_dim), s.q_rank)),
@@ -111,6 +113,7 @@ class LatentAttention(Mixer):
         self.w_uk_t = tensors[self._t("uk")].view(H, s.head_dim, s.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = tensors[self._t("uv")].view(H, s.value_dim, s.kv_rank).contiguous()
         self.w_o = runtime.weight(tensors[self._t("o")])
+        self.w_gate = runtime.weight(tensors[self._t("g")]) if getattr(s, "output_gate", False) else None
         d = int(s.rot_dim)
         self.inv_freq = None
         if d:
@@ -155,6 +158,11 @@ class LatentAttention(Mixer):
                                  cache.pools["latent"], cache.page_size, s.window, s.scale, chunk=s.chunk)
         heads_out = ctx.buffer("latent_heads", (n, H * s.value_dim), ctx.dtype)
         ops.gemm_batched(mixed, self.w_uv, heads_out, H, s.kv_rank, s.value_dim)
+        if self.w_gate is not None:
+            # the heads side by side times sigmoid(W_g x), x the mixer's own input
+            gate = ctx.buffer("latent_gate", (n, H * s.value_dim), ctx.dtype)
+            self.linear(x, self.w_gate, gate)
+            ops.gate_mul(heads_out, gate, heads_out)
         return self.linear_deferred(ctx, "attn_proj", heads_out, self.w_o)
 
 

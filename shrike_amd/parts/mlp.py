@@ -27,12 +27,18 @@ class SwiGLU(FeedForward):
         from ..kernels import ops
 
         ops.activation_code(self.spec.activation)  # raises for an activation the kernels lack
+        limit = getattr(self.spec, "limit", None)
+        if limit is not None and not limit > 0:
+            raise ValueError(f"{self.name}: limit must be positive, got {limit}")
 
     def load(self, tensors, runtime):
         self.inter = int(self.spec.intermediate_size)
         self.activation = self.spec.activation
+        self.limit = getattr(self.spec, "limit", None)
+        self.up_shift = float(getattr(self.spec, "up_shift", 0.0))
         self.w_gate_up = runtime.gated_weight(
-            tensors[self.tensor_name("gate", "gate_proj.weight")], tensors[self.tensor_name("up", "up_proj.weight")]
+            tensors[self.tensor_name("gate", "gate_proj.weight")], tensors[self.tensor_name("up", "up_proj.weight")],
+            self.activation, self.limit, self.up_shift,
         )
         self.w_down = runtime.weight(tensors[self.tensor_name("down", "down_proj.weight")])
         self.linear_deferred = runtime.linear_deferred
@@ -41,7 +47,7 @@ class SwiGLU(FeedForward):
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         n = x.shape[0]
         act = ctx.buffer("ffn_act", (n, self.inter), ctx.dtype)
-        self.gated_linear(ctx, x, self.w_gate_up, act, self.activation)
+        self.gated_linear(ctx, x, self.w_gate_up, act, self.activation, self.limit, self.up_shift)
         # the norm that follows adds the output to the residual stream and can add up parts
         return self.linear_deferred(ctx, "ffn_out", act, self.w_down)
 

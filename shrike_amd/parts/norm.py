@@ -39,6 +39,8 @@ class RMSNorm(Norm):
         else:
             ops.add_rmsnorm(hidden.resid, hidden.pending, self.weight, self.eps, out, rows, write_resid)
         if write_resid:
+            if hidden.pending is not None:
+                hidden.cast = None  # the stream has changed under a copy that an earlier kernel left
             hidden.pending = hidden.pending_norm = None
         return out
 
@@ -83,6 +85,8 @@ class LayerNorm(Norm):
                           weight=self.weight, bias=self.bias, eps=self.eps, out=out, rows=rows,
                           write_resid=write_resid, dtype=ctx.dtype)
         if write_resid:
+            if hidden.pending is not None:
+                hidden.cast = None  # the stream has changed under a copy that an earlier kernel left
             hidden.pending = hidden.pending_norm = None
         return out
 

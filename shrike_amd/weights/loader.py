@@ -54,7 +54,7 @@ def check_names(found: dict, params: list[ParamSpec]) -> None:
     wrong = sorted(
         (n, found[n][1], tuple(p.shape))
         for n, p in expected.items()
-        if n in found and tuple(found[n][1]) != tuple(p.shape)
+        if n in found and not p.matches(found[n][1])
     )
     if not (missing or unexpected or wrong):
         return

@@ -41,13 +41,14 @@ def random_tensor(p: ParamSpec, seed: int, dtype: torch.dtype, device="cpu",
                   mode: str = "reference") -> torch.Tensor:
     gen = torch.Generator(device=device)
     gen.manual_seed(_tensor_seed(seed, p.name))
+    shape = p.drawn_shape()
     try:
         std = _STD[p.init]
     except KeyError:
         raise ValueError(f"{p.name}: unknown init {p.init!r}") from None
     if mode == "unit":
         if p.init == "matrix":
-            std = float(p.shape[-1]) ** -0.5
+            std = float(shape[-1]) ** -0.5
         elif p.init == "embedding":
             std = 1.0
         elif p.init in ("bias", "vector"):
@@ -56,15 +57,15 @@ def random_tensor(p: ParamSpec, seed: int, dtype: torch.dtype, device="cpu",
             std = 0.2
     elif mode != "reference":
         raise ValueError(f"init mode must be one of {INIT_MODES}, got {mode!r}")
-    t = torch.empty(p.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+    t = torch.empty(shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
     if p.init == "norm":
         t += 1.0
     elif p.init == "positive":
         t = t.abs() + 0.01
     elif p.init == "near_identity":
-        t += torch.eye(p.shape[0], p.shape[1], device=device)
+        t += torch.eye(shape[0], shape[1], device=device)
     elif p.init == "average":
-        t += 1.0 / p.shape[0]
+        t += 1.0 / shape[0]
     return t.to(dtype)
 
 
