@@ -221,7 +221,7 @@ class PagedAttention(Mixer):
         if getattr(s, "bucket_bias", None):
             # (rows None: the table has as many rows as the file's tensor; random weights then draw 32)
             rows = s.bucket_bias[0]
-            out.append(ParamSpec(t("rel"), (None if rows is None else int(rows), s.num_heads), init="bias",
+            out.append(ParamSpec(t("rel"), (None if rows is None else int(rows), s.num_heads), init="score_bias",
                                  keep_float32=True, free_size=32))
         if getattr(s, "sinks", False):
             out.append(ParamSpec(t("sink"), (s.num_heads,), init="bias", keep_float32=True))

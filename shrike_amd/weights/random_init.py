@@ -24,7 +24,9 @@ from ..parts.base import ParamSpec
 _STD = {"matrix": 0.02, "embedding": 0.02, "bias": 0.02, "norm": 0.1, "norm_zero": 0.1, "vector": 0.02,
         # numbers that must be positive (|N(0, 0.5)| + 0.01), logarithms of rates, a square matrix
         # near the identity, and coefficients of an average (1 / count + N(0, 0.05))
-        "positive": 0.5, "log_rate": 0.5, "near_identity": 0.1, "average": 0.05}
+        "positive": 0.5, "log_rate": 0.5, "near_identity": 0.1, "average": 0.05,
+        # a table of numbers that are added to attention scores: N(0, 1) in both modes
+        "score_bias": 1.0}
 
 #: "reference": the distributions above.  "unit": matrices N(0, 1/fan_in) (the
 #: embedding table N(0, 1)), biases N(0, 0.1): every part's output is as large

@@ -220,3 +220,33 @@ def forward(cfg: dict, w: dict, tokens, return_layers: bool = False):
         streams.append(x)
     logits = (unit_rms(x, eps) * w["final.norm"]) @ w["embed"].T
     return (logits, torch.stack(streams)) if return_layers else logits
+
+
+class PlainPoresun:
+    """A model folder read once; `logits(ids)`, the stream after every layer, and greedy
+    generation over it, in float64 unless told otherwise."""
+
+    def __init__(self, model_dir, dtype=torch.float64):
+        import json
+        from pathlib import Path
+
+        from safetensors.torch import load_file
+
+        self.cfg = json.loads((Path(model_dir) / "config.json").read_text())
+        raw = load_file(str(Path(model_dir) / "model.safetensors"))
+        self.weights = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in raw.items()}
+
+    def logits(self, token_ids, rows=None) -> torch.Tensor:
+        out = forward(self.cfg, self.weights, list(token_ids))
+        return out if rows is None else out[torch.tensor(list(rows), dtype=torch.long)]
+
+    def layers(self, token_ids) -> torch.Tensor:
+        return forward(self.cfg, self.weights, list(token_ids), return_layers=True)[1]
+
+    def greedy(self, prompt, max_new_tokens: int) -> list[int]:
+        seq, out = list(prompt), []
+        for _ in range(max_new_tokens):
+            tok = int(torch.argmax(self.logits(seq)[-1]))
+            out.append(tok)
+            seq.append(tok)
+        return out

@@ -1,0 +1,263 @@
+"""The Poresun decoder in the engine against its plain implementation
+(tests/plain/poresun.py), on tiny models with random weights (tests/tiny_poresun.py):
+the stream after every layer; whole prompts, single tokens from the very first,
+portions down to two tokens and mixed batches over so few pages that they are used
+again (all pages that nobody holds poisoned with NaN); windows smaller than a page,
+across page edges and larger than any sequence; layers that read another layer's keys
+and values; long decoding; greedy generation through the entry point and its
+scheduler, with preemption; graphs and recorded launches against kernel-by-kernel
+steps; the command line."""
+
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from .compare import GreedyCheck
+from .plain.poresun import PlainPoresun
+from .tiny_poresun import CONFIGS, PAGE_SIZES, make_model_dir
+from .traces import (TraceBuilder, changing_portions, check_pages, last_one_by_one, mixed, read_pages,
+                     run_trace, whole)
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
+# lengths that end before, on and after the edges of the models' windows (5; 1, 37; 16, 1000),
+# of their bias tables' reach and of their pages
+LENGTHS = {"A": [1, 6, 49, 97, 130, 10], "B": [3, 41, 38, 29, 8, 150], "C": [2, 70, 17, 340]}
+
+
+@pytest.fixture(scope="module")
+def model_root(tmp_path_factory):
+    return tmp_path_factory.mktemp("poresun_models")
+
+
+def requests_for(name: str, lengths=None, seed: int = 0) -> dict[str, list[int]]:
+    rng = random.Random(sum(map(ord, name)) + seed)
+    vocab = CONFIGS[name]["vocab"]
+    return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(lengths or LENGTHS[name])}
+
+
+def engine_parts(model_dir, dtype, page_size, pages, graphs=True, slots=4):
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner
+
+    model, rt, _cfg = load_model(model_dir, dtype)
+    cache = CacheManager(model.cache_specs(), page_size, pages, max_slots=slots, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    return model, cache, ModelRunner(model, cache, rt, graphs=graphs)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_stream_after_every_layer(name, model_root):
+    """float32: the stream that every layer leaves against the plain model's, for a prompt
+    that crosses window edges."""
+    from shrike_amd.engine.runner import StepEntry
+    from shrike_amd.kernels import ops
+
+    model_dir = make_model_dir(name, model_root, dtype="float32")
+    plain = PlainPoresun(model_dir)
+    ids = requests_for(name, [75])["r0"]
+    want = plain.layers(ids)
+    model, cache, runner = engine_parts(model_dir, "float32", 16, 16, graphs=False)
+    seen = []
+    real = ops.postnorm
+
+    def watching(resid, *args, **kw):
+        real(resid, *args, **kw)
+        seen.append(resid.detach().cpu().double().clone())
+
+    ops.postnorm = watching
+    try:
+        seq = cache.new_sequence()
+        cache.append(seq, 0, len(ids))
+        runner.step([StepEntry(seq, ids, 0, [len(ids) - 1])])
+    finally:
+        ops.postnorm = real
+    sums = [2 if layer["mlp"] is not None else 1 for layer in CONFIGS[name]["layers"]]  # normed sums a layer
+    assert len(seen) == sum(sums) and want.shape[0] == len(sums)
+    at = -1
+    for run, (count, ref) in enumerate(zip(sums, want)):
+        at += count
+        err = float((seen[at] - ref).abs().max() / ref.abs().max())
+        assert err <= 2e-5, f"layer {run} ({CONFIGS[name]['layers'][run]['type']}): rel err {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, page_size", [("A", 16), ("B", 4), ("B", 16), ("C", 32), ("A", 8), ("C", 16)])
+def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtype, model_root, tmp_path):
+    model_dir = make_model_dir(name, model_root, dtype=dtype)
+    vocab = CONFIGS[name]["vocab"]
+    seqs = requests_for(name)
+    plain = PlainPoresun(model_dir)
+    want = {rid: plain.logits(ids).numpy() for rid, ids in seqs.items()}
+
+    tb = TraceBuilder()
+    budget = max(-(-len(ids) // 64) * 64 for ids in seqs.values())
+    whole(tb, "w_", seqs)
+    last_one_by_one(tb, "d_", seqs, tail=45)
+    changing_portions(tb, "p_", seqs)
+    mixed_budget = budget + 128
+    mixed(tb, "m_", seqs, mixed_budget, seed=5)
+    outputs = run_trace(model_dir, dtype, tb.steps, mixed_budget, tmp_path / "out", vocab,
+                        block_size=page_size, poison=True, pages=True)
+    got = tb.collect(outputs)
+    assert all(np.isfinite(rows).all() for rows in outputs.values()), "a page that nobody holds was read"
+    reused = check_pages(tb.steps, read_pages(tmp_path / "out", tb.steps), page_size, mixed_budget // page_size)
+    assert reused > 0, "the pool was meant to be so small that pages are used again"
+
+    scale = {rid: np.abs(w).max() for rid, w in want.items()}
+    worst, over = {}, []
+    for (rid, pos), row in got.items():
+        cut, name_ = rid.split("_", 1)
+        err = np.abs(row.astype(np.float64) - want[name_][pos]).max() / scale[name_]
+        worst[cut] = max(worst.get(cut, 0.0), err)
+        if err > TOL[dtype]:
+            over.append((rid, pos, err))
+    if dtype == "bfloat16":
+        # a router's close call now and then sends a token to another expert than the plain
+        # model's in bfloat16 (a jump, not a rounding: some of these models choose a single expert,
+        # and the norm after the sum carries the jump on undamped), in every cutting alike: few
+        # places, bounded
+        places = {(rid.split("_", 1)[1], pos) for rid, pos, _ in over}
+        assert len(places) <= 0.06 * sum(map(len, seqs.values())), over[:5]
+        assert all(e <= 1.0 for _, _, e in over), over[:5]
+    else:
+        assert not over, f"{over[0][0]} position {over[0][1]}: rel err {over[0][2]:.3e}"
+    assert set(worst) == {"w", "d", "p", "m"}
+    for cut in "wdp":
+        assert all((f"{cut}_{rid}", p) in got for rid, ids in seqs.items() for p in range(len(ids)))
+    if dtype == "float32":  # every float32 kernel sums a row in one order whatever the step holds
+        for (rid, pos), row in got.items():
+            cut, name_ = rid.split("_", 1)
+            assert np.array_equal(row, got[(f"w_{name_}", pos)]), f"{rid} position {pos} differs from the whole prompt's"
+    print(f"{name} page {page_size} {dtype}: worst rel err per cutting {worst}, {len(over)} of {len(got)} rows over")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding_from_the_first_token(name, model_root):
+    """Every token on the single-token path (graphs included), the windows passing over
+    decoded tokens; pages that a window has passed are given back on the way, but not those
+    of a windowed layer whose cache a causal layer reads."""
+    from shrike_amd.engine.runner import StepEntry
+
+    for dtype, tol in TOL.items():
+        model_dir = make_model_dir(name, model_root, dtype=dtype)
+        plain = PlainPoresun(model_dir)
+        page = PAGE_SIZES[name]
+        model, cache, runner = engine_parts(model_dir, dtype, page, 64)
+        ids = requests_for(name, [230], seed=3)["r0"]
+        want = plain.logits(ids)
+        seq = cache.new_sequence()
+        rows = []
+        for p, tok in enumerate(ids):
+            cache.append(seq, p, 1)
+            rows.append(runner.step([StepEntry(seq, [tok], p, [0])]).cpu().clone())
+            cache.trim(seq, p + 1)
+        got = torch.cat(rows).double()
+        err = (got - want).abs().amax(-1) / want.abs().max()
+        if dtype == "bfloat16":
+            assert float((err > tol).float().mean()) <= 0.06 and float(err.max()) <= 1.0, \
+                f"bfloat16: {int((err > tol).sum())} positions over {tol}, worst {float(err.max()):.3e}"
+        else:
+            assert float(err.max()) <= tol, f"{dtype}: worst at position {int(err.argmax())}: {float(err.max()):.3e}"
+        windows = [g.spec.window for g in cache.groups]
+        assert any(w is not None for w in windows)
+        for g, table in zip(cache.groups, seq.tables):
+            if g.spec.window is not None:
+                assert sum(x >= 0 for x in table) <= -(-g.spec.window // page) + 1, "pages behind the window were kept"
+            else:
+                assert all(x >= 0 for x in table[: -(-len(ids) // page)])
+        assert runner.graph_replays > 100
+        cache.free(seq)
+        cache.check([])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, lengths, new, budget", [("A", [1, 20, 47, 30], 60, 16), ("B", [5, 13, 2], 30, 512),
+                                                        ("C", [40, 3], 25, 24)])
+def test_greedy_generation_through_the_entry_point(name, lengths, new, budget, dtype, model_root):
+    """Prompts in portions under a small token budget beside decoding requests, through
+    LLM.generate and its scheduler; float32: the plain model's greedy tokens exactly."""
+    from shrike_amd import LLM, SamplingParams
+
+    if dtype == "bfloat16" and name == "B":
+        # a router's close call in bfloat16 moves a logit by more than rounding does (this model's
+        # last layer sends a token to a single expert): its tokens are compared in float32
+        pytest.skip("greedy tokens of this model are compared in float32 only")
+    model_dir = make_model_dir(name, model_root, dtype=dtype)
+    plain = PlainPoresun(model_dir)
+    prompts = list(requests_for(name, lengths, seed=9).values())
+    llm = LLM(str(model_dir), dtype=dtype, block_size=PAGE_SIZES[name], num_kv_blocks=96, max_tokens_per_step=budget)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
+    assert [len(o) for o in outs] == [new] * len(prompts)
+    check = GreedyCheck(plain, dtype)
+    for prompt, out in zip(prompts, outs):
+        check.request(prompt, out)
+    check.finish()
+    assert llm.engine.cache.num_free == llm.engine.cache.num_pages
+
+
+def test_generation_survives_preemption_when_pages_run_out(model_root):
+    """So few pages that the newest request is preempted, gives its pages back and recomputes
+    from its first token: the tokens are the plain model's all the same."""
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir("A", model_root, dtype="float32")
+    plain = PlainPoresun(model_dir)
+    prompts = list(requests_for("A", [30, 28, 33], seed=2).values())
+    llm = LLM(str(model_dir), dtype="float32", block_size=16, num_kv_blocks=9, max_tokens_per_step=64)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=40, ignore_eos=True))
+    assert llm.engine.metrics()["preemptions"] > 0
+    for prompt, out in zip(prompts, outs):
+        assert out == plain.greedy(prompt, 40)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_graphs_and_recorded_launches_equal_kernel_by_kernel_steps(name, dtype, model_root):
+    """The same steps with and without HIP graphs and recorded launch lists: the same bits."""
+    from shrike_amd.engine.runner import StepEntry
+
+    model_dir = make_model_dir(name, model_root, dtype=dtype)
+    ids = requests_for(name, [90, 41], seed=4)
+    results = []
+    for graphs in (True, False):
+        model, cache, runner = engine_parts(model_dir, dtype, 16, 32, graphs=graphs)
+        a, b = cache.new_sequence(), cache.new_sequence()
+        rows = []
+        pa = pb = 0
+        for step in range(40):
+            entries = []
+            na = 7 if pa < 60 else 1  # portions of a first, then single tokens
+            na = min(na, len(ids["r0"]) - pa)
+            if na:
+                cache.append(a, pa, na)
+                entries.append(StepEntry(a, ids["r0"][pa : pa + na], pa, [na - 1]))
+            nb = 1 if pb < len(ids["r1"]) else 0
+            if nb:
+                cache.append(b, pb, 1)
+                entries.append(StepEntry(b, [ids["r1"][pb]], pb, [0]))
+            if not entries:
+                break
+            rows.append(runner.step(entries).cpu().clone())
+            pa, pb = pa + na, pb + nb
+            cache.trim(a, pa), cache.trim(b, pb)
+        if graphs:
+            assert runner.graph_replays > 0 and runner.list_replays > 0
+        results.append(torch.cat(rows))
+    assert torch.equal(results[0], results[1])
+
+
+def test_command_line_generates_with_a_model_folder(model_root, capsys):
+    from shrike_amd.__main__ import main
+
+    model_dir = make_model_dir("A", model_root, dtype="float32")
+    rc = main(["--model", str(model_dir), "--prompt-ids", "5,6,7,8,140,2", "--max-tokens", "9", "--dtype", "fp32",
+               "--block-size", "4", "--num-kv-blocks", "16", "--ignore-eos", "--metrics"])
+    assert rc == 0
+    out = capsys.readouterr()
+    assert [int(t) for t in out.out.split()] == PlainPoresun(model_dir).greedy([5, 6, 7, 8, 140, 2], 9)
+    assert "tokens_generated" in out.err
