@@ -198,13 +198,13 @@ int shk_attention_supports_mfma(int heads, int kv_heads, int head_dim, int page_
 // `partial` is float32 scratch of num_seqs * heads * nsplit * (head_dim + 2).
 // streaming != 0: keys and values are fetched with non-temporal loads (faster when a
 // launch reads tens of megabytes of them, slightly slower below; the result is the same).
-// softcap / sinks as in shk_attention (0 and null: neither).
+// softcap / sinks / dist_bias as in shk_attention (0 and null: none).
 int shk_attention_decode_bf16(const void* q, int q_stride, void* out, int num_seqs, int heads,
                               int kv_heads, int head_dim, const int32_t* positions,
                               const int32_t* tables, int table_stride, const void* k_pool,
                               const void* v_pool, int page_size, int window, int chunk, float scale,
                               float* partial, int nsplit, int streaming, float softcap, const float* sinks,
-                              void* stream);
+                              const float* dist_bias, int bias_rows, void* stream);
 
 // bfloat16 attention for prompt portions, in tiles of 16 queries: tile i covers
 // queries tile_q0[i] .. +16 of sequence tile_seq[i]'s portion.  cu_q[s] is the
@@ -237,7 +237,8 @@ int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out, in
                                       int table_stride, const void* k_pool, const void* v_pool,
                                       int page_size, int window, int chunk, float scale, int small,
                                       float* partial, int nsplit, int first_token,
-                                      int prompt_tokens, float softcap, const float* sinks, void* stream);
+                                      int prompt_tokens, float softcap, const float* sinks,
+                                      const float* dist_bias, int bias_rows, void* stream);
 
 // Attention through latents (latent.hip).  shk_latent_prepare: `down` is [n, q_rank +
 // kv_rank + rot_dim], a token's joint down-projection; q_latent [n, q_rank] receives

@@ -84,11 +84,28 @@ __device__ __forceinline__ float lanes4_sum(float v) {
 //   cap_out != 0: s <- cap * tanh(s * scale / cap), formed as cap_out * (1 - 2 / (1 + 2^(s * cap_in)))
 //                 with cap_in = 2 * scale * log2(e) / cap and cap_out = cap * log2(e);
 //   sinks != null: one more term 2^(sinks[head] * log2(e)) in the head's denominator, which has
-//                 no key and no value (added where a row is normalised, or by the merge kernel).
+//                 no key and no value (added where a row is normalised, or by the merge kernel);
+//   dist_bias != null: a learned number per head and distance, dist_bias[head][min(i - j, bias_rows - 1)],
+//                 joins the (capped) score.
 struct ScoreOpts {
   float cap_in, cap_out;
   const float* sinks;
+  const float* dist_bias;
+  int bias_rows;
 };
+
+// The eight scores (base-2 logarithms) of a lane's keys key0 .. key0 + 7 for the query at `pos`, each plus
+// its head's bias for the distance; keys that the query does not read (masked afterwards) take any row.
+__device__ __forceinline__ void add_distance_bias(float (&sc)[8], const ScoreOpts& so, int head, int pos, int key0) {
+  const float* row = so.dist_bias + static_cast<size_t>(head) * so.bias_rows;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    int d = pos - (key0 + e);
+    d = d < 0 ? 0 : d;
+    d = d < so.bias_rows ? d : so.bias_rows - 1;
+    sc[e] = fmaf(row[d], 1.4426950408889634f, sc[e]);
+  }
+}
 
 __device__ __forceinline__ float capped_log2(float s, const ScoreOpts& so) {
   return so.cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(s * so.cap_in)));
@@ -469,6 +486,10 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
         for (int e = 0; e < 8; ++e) sc[e] = capped_log2(s[e / 4][e % 4], so);
       }
       const int g0 = kb + g * 8;
+      if (so.dist_bias) {  // (the same for every wavefront of the launch)
+        asm volatile("");
+        add_distance_bias(sc, so, kvh * group + (j < group ? j : group - 1), pos, g0);
+      }
       if (edge) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -932,6 +953,10 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
 #pragma unroll
         for (int e = 0; e < 8; ++e) sc[e] = capped_log2(s[e / 4][e % 4], so);
       }
+      if (so.dist_bias) {  // (the same for every wavefront of the launch)
+        asm volatile("");
+        add_distance_bias(sc, so, unit_head[u] < heads ? unit_head[u] : heads - 1, q_pos[u], g0);
+      }
       if (edge) {  // wave-uniform: some query of the workgroup does not read the whole chunk
         // (the empty statement keeps this a branch: turned into selects, the
         // comparisons would run for every chunk)
@@ -1087,10 +1112,10 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
         partial, out + static_cast<size_t>(first_token) * heads * D, nsplit, so.sinks, heads);
 }
 
-static ScoreOpts score_opts(float scale, float softcap, const float* sinks) {
+static ScoreOpts score_opts(float scale, float softcap, const float* sinks, const float* dist_bias, int bias_rows) {
   const float log2e = 1.4426950408889634f;
-  if (softcap > 0.f) return ScoreOpts{2.f * scale * log2e / softcap, softcap * log2e, sinks};
-  return ScoreOpts{0.f, 0.f, sinks};
+  if (softcap > 0.f) return ScoreOpts{2.f * scale * log2e / softcap, softcap * log2e, sinks, dist_bias, bias_rows};
+  return ScoreOpts{0.f, 0.f, sinks, dist_bias, bias_rows};
 }
 
 }  // namespace shk
@@ -1135,9 +1160,10 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
                                          int table_stride, const void* k_pool, const void* v_pool,
                                          int page_size, int window, int block, float scale, float* partial,
                                          int nsplit, int streaming, float softcap, const float* sinks,
-                                         void* stream) {
+                                         const float* dist_bias, int bias_rows, void* stream) {
   SHK_REQUIRE(softcap >= 0.f, "attention_decode: a score cap must be positive (0: none), got %g", softcap);
-  const ScoreOpts so = score_opts(scale, softcap, sinks);
+  SHK_REQUIRE(!dist_bias || bias_rows > 0, "attention_decode: a distance bias needs a table of at least one row");
+  const ScoreOpts so = score_opts(scale, softcap, sinks, dist_bias, bias_rows);
   if (check_mfma_shapes("attention_decode", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
   SHK_REQUIRE(heads / kv_heads <= 16, "attention_decode: at most 16 query heads per key/value head");
   SHK_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && nsplit >= 1 && nsplit <= kMaxSplits,
@@ -1183,9 +1209,12 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
                                                  const void* v_pool, int page_size, int window, int block,
                                                  float scale, int small, float* partial, int nsplit,
                                                  int first_token, int prompt_tokens, float softcap,
-                                                 const float* sinks, void* stream) {
+                                                 const float* sinks, const float* dist_bias, int bias_rows,
+                                                 void* stream) {
   SHK_REQUIRE(softcap >= 0.f, "attention_prefill_shared: a score cap must be positive (0: none), got %g", softcap);
-  const ScoreOpts so = score_opts(scale, softcap, sinks);
+  SHK_REQUIRE(!dist_bias || bias_rows > 0,
+              "attention_prefill_shared: a distance bias needs a table of at least one row");
+  const ScoreOpts so = score_opts(scale, softcap, sinks, dist_bias, bias_rows);
   if (check_mfma_shapes("attention_prefill_shared", heads, kv_heads, head_dim, page_size, q_stride))
     return 1;
   const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim, small);

@@ -531,6 +531,12 @@ def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k
     )
 
 
+def _dist_bias_args(dist_bias, heads, who):
+    """(address, rows) of a distance bias for a launcher; (None, 0) without one."""
+    _dist_bias(dist_bias, heads, who)
+    return (None, 0) if dist_bias is None else (_dev(dist_bias, "dist_bias", torch.float32), dist_bias.shape[1])
+
+
 def _dist_bias(dist_bias, heads, who):
     if dist_bias is not None and (dist_bias.dim() != 2 or dist_bias.shape[0] != heads or dist_bias.shape[1] < 1
                                   or not dist_bias.is_contiguous() or dist_bias.dtype != torch.float32):
@@ -1109,7 +1115,7 @@ def _sinks(sinks, heads, who):
 
 def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tables, k_pool, v_pool,
                      page_size, window, scale, partial, nsplit, streaming=False, chunk=None, softcap=None,
-                     sinks=None) -> None:
+                     sinks=None, dist_bias=None) -> None:
     """bfloat16 MFMA attention for the first num_seqs rows of q, one token per sequence.
     `streaming`: fetch keys and values with non-temporal loads (same result; faster when
     the launch reads tens of megabytes of them)."""
@@ -1129,7 +1135,8 @@ def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tab
             _dev(positions, "positions", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size,
             int(window or 0), int(chunk or 0), float(scale), _dev(partial, "partial", torch.float32), nsplit,
-            int(bool(streaming)), float(softcap or 0.0), _sinks(sinks, heads, "attention_decode"), _stream(),
+            int(bool(streaming)), float(softcap or 0.0), _sinks(sinks, heads, "attention_decode"),
+            *_dist_bias_args(dist_bias, heads, "attention_decode"), _stream(),
         )
     )
 
@@ -1165,7 +1172,7 @@ def attention_prefill_shared_tiles(heads, kv_heads, head_dim, small=False) -> in
 def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, ctx_lens, wg_seq, wg_q0,
                              tables, k_pool, v_pool, page_size, window, scale, small=False,
                              partial=None, nsplit: int = 1, first_token: int = 0, chunk=None, softcap=None,
-                             sinks=None) -> None:
+                             sinks=None, dist_bias=None) -> None:
     """bfloat16 MFMA attention for prompt portions; one workgroup per (run of query
     tiles, key/value head) shares each chunk of keys among its query heads.
     wg_seq / wg_q0 are in steps of 16 * attention_prefill_shared_tiles(..., small),
@@ -1194,7 +1201,8 @@ def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, c
             _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
             _dev(v_pool, "v_pool"), page_size, int(window or 0), int(chunk or 0), float(scale), int(small),
             _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), int(first_token),
-            int(prompt_tokens), float(softcap or 0.0), _sinks(sinks, heads, "attention_prefill_shared"), _stream(),
+            int(prompt_tokens), float(softcap or 0.0), _sinks(sinks, heads, "attention_prefill_shared"),
+            *_dist_bias_args(dist_bias, heads, "attention_prefill_shared"), _stream(),
         )
     )
 

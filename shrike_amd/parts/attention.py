@@ -380,11 +380,9 @@ class PagedAttention(Mixer):
             return
         plan.mfma = self.dtype == torch.bfloat16 and self.value_dim == d and ops.attention_supports_mfma(
             h, hkv, d, shape.page_size, self._qkv_width())
-        if getattr(s, "bucket_bias", None):
-            plan.mfma = False
-        # capped scores and sinks are built into the decode kernel and the shared-key prompt
+        # capped scores, sinks and a bias table are built into the decode kernel and the shared-key prompt
         # kernel; where the latter does not take the shape, the general kernel serves the step
-        if plan.mfma and (getattr(s, "softcap", None) or getattr(s, "sinks", False)) \
+        if plan.mfma and (getattr(s, "softcap", None) or getattr(s, "sinks", False) or getattr(s, "bucket_bias", None)) \
                 and not ops.attention_prefill_shared_tiles(h, hkv, d):
             plan.mfma = False
         # the most keys that any query reads, where the mask bounds them
@@ -428,7 +426,7 @@ class PagedAttention(Mixer):
         plan.count = int(seqs.size)
         # what the launches of the portions depend on beyond the step's sizes
         shape.launch_key.append((key, plan.kernel, plan.small, plan.portion_splits, plan.first_token, plan.count))
-        tag = f"{h}:{hkv}:{d}:{s.window or 0}:{s.chunk or 0}"
+        tag = ":".join(str(int(x or 0)) for x in key[1:])  # (one list per plan: the plan's key names it)
         plan.seq_name, plan.q0_name = f"attention_seq:{tag}", f"attention_q0:{tag}"
         shape.add(plan.seq_name, seqs)
         shape.add(plan.q0_name, q0)
@@ -473,7 +471,7 @@ class PagedAttention(Mixer):
             ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale,
                                  partial, plan.nsplit, plan.streaming, chunk=s.chunk,
-                                 softcap=getattr(s, "softcap", None), sinks=self.sinks)
+                                 softcap=getattr(s, "softcap", None), sinks=self.sinks, dist_bias=self.dist_bias)
         if plan.kernel == "shared":
             partial = None
             if plan.portion_splits > 1:
@@ -485,7 +483,8 @@ class PagedAttention(Mixer):
                                          cache.pools["k"], cache.pools["v"], cache.page_size, s.window,
                                          s.scale, small=plan.small, partial=partial,
                                          nsplit=plan.portion_splits, first_token=plan.first_token,
-                                         chunk=s.chunk, softcap=getattr(s, "softcap", None), sinks=self.sinks)
+                                         chunk=s.chunk, softcap=getattr(s, "softcap", None), sinks=self.sinks,
+                                         dist_bias=self.dist_bias)
         elif plan.kernel == "tiles":
             ops.attention_prefill(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                   ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
