@@ -327,7 +327,8 @@ def kernel_breakdown(engine, steps: int = 3, before_step=None) -> dict:
              "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows", "embed_pairs", "qkv_store",
              "latent_prepare", "rotate_heads", "latent_attention", "latent_attention_mfma", "gemm_batched", "mlstm_scan", "headnorm_gate",
              "xielu", "layernorm", "add_layernorm", "attention_talking", "attention_talking_mfma", "conv_silu", "dt_softplus", "selective_scan",
-             "rotate_half_rows", "retention_scan", "moe_route", "moe_experts", "mix_history", "scale_softcap"]
+             "rotate_half_rows", "retention_scan", "moe_route", "moe_experts", "mix_history", "scale_softcap",
+             "postnorm", "cast_rows", "activate", "gate_mul"]
     names = [n for n in names if hasattr(ops, n)]
     spans: list[tuple[str, object, object]] = []
     saved = {n: getattr(ops, n) for n in names}
@@ -510,6 +511,81 @@ def ligipel_like(qcfg, window: int, pattern: str, experts: int, top: int):
     return lcfg, sizes
 
 
+def poresun_like(qcfg, window: int, pattern: str, experts: int, top: int):
+    """A Poresun configuration with the layer sizes of a Qwen2 one (same width, vocabulary and
+    number of layers).  `pattern` says which mixer each layer has, letter by letter, repeated:
+    a, attention with Qwen2's heads, unweighted norms of queries and keys, a cap, a bias table
+    of 32 rows that reaches 4,096 positions and a sliding window `window`; b, the causal
+    attention with weighted norms, a query temperature and the same table; s, such a layer
+    that reads the keys and values of the last b layer before it; l, latent attention with as
+    many heads, a query latent of 3/8 and a key/value latent of 1/8 of the width (rounded to
+    64), half a head rotated, and the output gate.  The first layer of every repetition has the
+    bounded gated feed-forward as wide as Qwen2's; the others `experts` routed experts without
+    gates of which a token uses `top` (together half of Qwen2's feed-forward's multiply-adds)
+    and a gated shared expert of the other half.  With it an object that names the sizes as the
+    formulas of this program expect them (see ligipel_like)."""
+    from types import SimpleNamespace
+
+    from shrike_amd.models.poresun import (BoundedDense, BucketAttention, GatedLatentAttention, PoresunConfig,
+                                           PoresunLayer, UngatedMixture)
+
+    h, d, H, KV = qcfg.hidden_size, qcfg.head_dim, qcfg.num_attention_heads, qcfg.num_key_value_heads
+    inter = qcfg.intermediate_size
+    up64 = lambda x: max(64, -(-int(x) // 64) * 64)  # noqa: E731
+    # an expert has two matrices where Qwen2's feed-forward has three
+    ff = max(64, 3 * inter // (4 * top) // 64 * 64)
+    shared = up64(3 * inter / 4)
+    latent = GatedLatentAttention(heads=H, dim=d, rot_dim=d // 2, vdim=d, q_rank=up64(3 * h / 8), kv_rank=up64(h / 8),
+                                  scale=(1.5 * d) ** -0.5, rot_base=10000.0, rot_dims=d // 2)
+    layers, last_b = [], None
+    for i in range(qcfg.num_hidden_layers):
+        letter = pattern[i % len(pattern)]
+        if letter == "s" and last_b is None:
+            letter = "b"
+        if letter == "a":
+            kind, mixer = "attention", BucketAttention(heads=H, kv_heads=KV, dim=d, vdim=d, scale=d**-0.5, bias_max=4096,
+                                                       weighted_norm=False, window=window, softcap=30.0, bias_rows=32)
+        elif letter in "bs":
+            kind, mixer = "attention_2", BucketAttention(heads=H, kv_heads=KV, dim=d, vdim=d, scale=d**-0.5, bias_max=4096,
+                                                         weighted_norm=True, q_temp=(0.25, 256), bias_rows=32,
+                                                         kv_from=last_b if letter == "s" else None)
+            last_b = i if letter == "b" else last_b
+        elif letter == "l":
+            kind, mixer = "latent_attention", latent
+        else:
+            raise SystemExit(f"--pattern: unknown letter {letter!r} for --poresun (a, b, s, l)")
+        mlp = BoundedDense(ff=inter, limit=7.0) if i % len(pattern) == 0 else \
+            UngatedMixture(experts=experts, top=top, ff=ff, shared_ff=shared)
+        layers.append((letter, PoresunLayer(kind, mixer, mlp)))
+    pcfg = PoresunConfig(vocab=qcfg.vocab_size, width=h, norm_eps=qcfg.rms_norm_eps, alpha=2.0,
+                         layers=tuple(layer for _, layer in layers), embedding_scale=float(h) ** 0.5)
+    n = len(layers)
+    mixer_elements = {
+        "a": 2 * (H + KV) * d * h, "b": 2 * (H + KV) * d * h, "s": 2 * H * d * h,
+        "l": (latent.q_rank + latent.kv_rank + latent.rot_dim) * h + H * (d + latent.rot_dim) * latent.q_rank
+        + 2 * H * d * latent.kv_rank + 2 * H * d * h,
+    }
+    cached = {"a": 2 * KV * d, "b": 2 * KV * d, "s": 0, "l": latent.kv_rank + latent.rot_dim}
+    dense_layers = sum(isinstance(layer.mlp, BoundedDense) for _, layer in layers)
+    mixers = sum(mixer_elements[letter] for letter, _ in layers)
+    sizes = SimpleNamespace(
+        hidden_size=h, head_dim=d, num_attention_heads=H, num_key_value_heads=KV, intermediate_size=inter,
+        num_hidden_layers=n, vocab_size=qcfg.vocab_size, attention_layers=sum(letter != "l" for letter, _ in layers),
+        kv_elements_per_token=sum(cached[letter] for letter, _ in layers))
+
+    def elements(per_expert_layer: float) -> int:
+        moe = (experts + 1) * h + 2 * h * shared + per_expert_layer
+        return int((mixers + dense_layers * 3 * h * inter + (n - dense_layers) * moe) // n)
+
+    def at_batch(b: int) -> None:
+        touched = experts * (1.0 - (1.0 - top / experts) ** b)
+        sizes.layer_elements = elements(touched * 2 * h * ff)
+
+    sizes.at_batch = at_batch
+    sizes.layer_elements = elements(top * 2 * h * ff)  # a prompt: every token's own experts are work
+    return pcfg, sizes
+
+
 def run_designs(args, qcfg) -> dict:
     """Another design beside Qwen2 at equal layer sizes, random weights: a prompt of 2,048
     tokens in one step, decode steps at batch 1, 8 and 64 from that context, and what each
@@ -519,9 +595,13 @@ def run_designs(args, qcfg) -> dict:
     import torch
 
     from shrike_amd import SamplingParams
-    from shrike_amd.models import ligipel, minilorn, mofarax, qwen2
+    from shrike_amd.models import ligipel, minilorn, mofarax, poresun, qwen2
 
-    if args.ligipel:
+    if args.poresun:
+        pcfg, psizes = poresun_like(qcfg, args.window, args.pattern if set(args.pattern) <= set("absl") else "absl",
+                                    args.experts, args.top)
+        other = ("poresun", poresun.build_spec(pcfg), psizes)
+    elif args.ligipel:
         lcfg, lsizes = ligipel_like(qcfg, args.window, args.pattern if set(args.pattern) <= set("pr") else "pppr",
                                     args.experts, args.top)
         other = ("ligipel", ligipel.build_spec(lcfg), lsizes)
@@ -711,15 +791,20 @@ def main() -> int:
                     help="Minilorn beside Qwen2 at equal layer sizes: prompt, decode at batch 1/8/64, time per kernel")
     ap.add_argument("--ligipel", action="store_true",
                     help="Ligipel beside Qwen2 at equal layer sizes: prompt, decode at batch 1/8/64, time per kernel")
-    ap.add_argument("--experts", type=int, default=8, metavar="N", help="--ligipel: routed experts a layer")
-    ap.add_argument("--top", type=int, default=2, metavar="N", help="--ligipel: experts a token uses")
+    ap.add_argument("--poresun", action="store_true",
+                    help="the Poresun design beside Qwen2 at the layer sizes of --shape, random weights")
+    ap.add_argument("--experts", type=int, default=8, metavar="N", help="--ligipel, --poresun: routed experts a layer")
+    ap.add_argument("--top", type=int, default=2, metavar="N", help="--ligipel, --poresun: experts a token uses")
     ap.add_argument("--pattern", default="alml", metavar="LETTERS",
                     help="--minilorn: the layers' mixers in order, repeated: a(ttention), l(atent attention), m(atrix memory); "
-                         "--ligipel: p(arallel attention and scan), r(etention), default pppr")
+                         "--ligipel: p(arallel attention and scan), r(etention), default pppr; --poresun: a(ttention "
+                         "with a window), b (causal attention), s (reads the last b layer's keys and values), "
+                         "l(atent attention), default absl")
     ap.add_argument("--window", type=int, default=4096, metavar="N",
                     help="--minilorn: sliding window of its latent attention (4096: no fewer keys than Qwen2 reads)")
-    ap.add_argument("--design-only", choices=["qwen2", "mofarax", "minilorn", "ligipel"], default=None,
-                    help="--mofarax / --minilorn / --ligipel: run only this one of the two (for a profile of one model's kernels)")
+    ap.add_argument("--design-only", choices=["qwen2", "mofarax", "minilorn", "ligipel", "poresun"], default=None,
+                    help="--mofarax / --minilorn / --ligipel / --poresun: run only this one of the two (for a profile of "
+                         "one model's kernels)")
     ap.add_argument("--mask-size", type=int, default=8192, metavar="N",
                     help="--mofarax: positions per block of its attention (8192: no fewer keys than Qwen2 reads)")
     ap.add_argument("--side-dim", type=int, default=256, metavar="N", help="--mofarax: width of its per-layer token input")
@@ -752,13 +837,15 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
-    if args.mofarax or args.minilorn or args.ligipel:
+    if args.mofarax or args.minilorn or args.ligipel or args.poresun:
         designs = run_designs(args, cfg)
-        design = "Ligipel" if args.ligipel else "Minilorn" if args.minilorn else "Mofarax"
+        design = "Poresun" if args.poresun else "Ligipel" if args.ligipel else "Minilorn" if args.minilorn else "Mofarax"
         config = {"shape": args.shape, "layers": cfg.num_hidden_layers, "prompt": PROMPT_LEN,
                   "decode_steps": args.design_steps}
-        config.update({"pattern": args.pattern if set(args.pattern) <= set("pr") else "pppr", "window": args.window,
-                       "experts": args.experts, "top": args.top} if args.ligipel
+        config.update({"pattern": args.pattern if set(args.pattern) <= set("absl") else "absl", "window": args.window,
+                       "experts": args.experts, "top": args.top} if args.poresun
+                      else {"pattern": args.pattern if set(args.pattern) <= set("pr") else "pppr", "window": args.window,
+                            "experts": args.experts, "top": args.top} if args.ligipel
                       else {"pattern": args.pattern, "window": args.window} if args.minilorn
                       else {"mask_size": args.mask_size, "side_dim": args.side_dim})
         print(json.dumps({

@@ -147,12 +147,17 @@ __global__ void __launch_bounds__(256)
     const T* gr = wg + (static_cast<size_t>(e) * ff + f) * width;
     const T* ur = wu + (static_cast<size_t>(e) * ff + f) * width;
     float g = 0.f, u = 0.f;
-    for (int k = lane; k < width; k += kWave) {
-      g = fmaf(to_float(gr[k]), xs[k], g);
-      u = fmaf(to_float(ur[k]), xs[k], u);
+    if (wg == wu) {  // experts without a gate: the one product is both factors
+      for (int k = lane; k < width; k += kWave) g = fmaf(to_float(gr[k]), xs[k], g);
+      g = u = wave_sum(g);
+    } else {
+      for (int k = lane; k < width; k += kWave) {
+        g = fmaf(to_float(gr[k]), xs[k], g);
+        u = fmaf(to_float(ur[k]), xs[k], u);
+      }
+      g = wave_sum(g);
+      u = wave_sum(u);
     }
-    g = wave_sum(g);
-    u = wave_sum(u);
     if (lane == 0) act_out[static_cast<size_t>(pair) * ff + f] = from_float<T>(gate_act(g, act) * u);
   }
 }
@@ -231,6 +236,7 @@ __global__ void __launch_bounds__(256)
   const int count = min(counts[e], n);
   const int row0 = blockIdx.y * 32;
   if (row0 >= count) return;
+  const bool single = wg == wu;  // experts without a gate: the one product is both factors
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int i = lane % 16, kg = lane / 16;
   const int f0 = (blockIdx.x * 4 + wave) * 32;
@@ -263,7 +269,7 @@ __global__ void __launch_bounds__(256)
       if (have) {
         if (pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(xr[a] + k0);
         gv[a] = *reinterpret_cast<const uint4*>(gr[a] + k0);
-        uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
+        if (!single) uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
       }
     }
 #pragma unroll
@@ -272,8 +278,9 @@ __global__ void __launch_bounds__(256)
       for (int b = 0; b < 2; ++b) {
         accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, gv[b]),
                                                              __builtin_bit_cast(mbf16x8, av[a]), accg[a][b], 0, 0, 0);
-        accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
-                                                             __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
+        if (!single)
+          accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
+                                                               __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
       }
   }
   // features were the rows of the products: this lane holds features f0 + 16 b + 4 kg + r of pair row a * 16 + i
@@ -286,7 +293,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int f = f0 + b * 16 + 4 * kg + r;
-        if (f < ff) dst[f] = from_float<bf16>(gate_act(accg[a][b][r], act) * accu[a][b][r]);
+        if (f < ff) dst[f] = from_float<bf16>(gate_act(accg[a][b][r], act) * (single ? accg[a][b][r] : accu[a][b][r]));
       }
   }
 }
@@ -371,7 +378,9 @@ __global__ void __launch_bounds__(256)
 constexpr int kTileRows = 128;
 constexpr int kTileLd = 40;  // elements between rows in LDS (32 and 16 bytes of padding)
 
-template <bool GATED>
+// SINGLE (with GATED): the experts have no gate; the tile is 128 features of the one matrix, as in the
+// down product, over the tokens' rows, and a feature's product is both factors of its activation.
+template <bool GATED, bool SINGLE = false>
 __global__ void __launch_bounds__(256)
     moe_tiled_mfma_kernel(const bf16* __restrict__ a, const int32_t* __restrict__ order,
                           const int32_t* __restrict__ counts, const bf16* __restrict__ w0, const bf16* __restrict__ w1,
@@ -395,7 +404,7 @@ __global__ void __launch_bounds__(256)
     const int pair = r < count ? list[r] : -1;
     // gate/up: a pair's row is its token's; down: its own row of activations
     arow[h] = pair < 0 ? nullptr : a + static_cast<size_t>(GATED ? min(pair / top, n - 1) : min(pair, n * top - 1)) * k + lp * 8;
-    if (GATED) {
+    if (GATED && !SINGLE) {
       const int f = blockIdx.x * 64 + lr;
       brow[h] = f < m ? (h == 0 ? w0 : w1) + (static_cast<size_t>(e) * m + f) * k + lp * 8 : nullptr;
     } else {
@@ -420,6 +429,7 @@ __global__ void __launch_bounds__(256)
       *reinterpret_cast<uint4*>(&sb[buf][(lr + 64 * h) * kTileLd + lp * 8]) = rb[h];
     }
   };
+  constexpr int kOperands = 4;  // B operands a step
   mf32x4 acc[4][4];
 #pragma unroll
   for (int am = 0; am < 4; ++am)
@@ -437,15 +447,15 @@ __global__ void __launch_bounds__(256)
     for (int am = 0; am < 4; ++am)
       af[am] = __builtin_bit_cast(mbf16x8, *reinterpret_cast<const uint4*>(&sa[buf][(wm * 64 + am * 16 + i) * kTileLd + kg * 8]));
 #pragma unroll
-    for (int bn = 0; bn < 4; ++bn) {
+    for (int bn = 0; bn < kOperands; ++bn) {
       // gate/up: operands 0, 1 are this wavefront's 32 gate features, 2, 3 the same features of up (rows 64 on)
-      const int brw = GATED ? (bn / 2) * 64 + wn * 32 + (bn % 2) * 16 + i : wn * 64 + bn * 16 + i;
+      const int brw = GATED && !SINGLE ? (bn / 2) * 64 + wn * 32 + (bn % 2) * 16 + i : wn * 64 + bn * 16 + i;
       bf[bn] = __builtin_bit_cast(mbf16x8, *reinterpret_cast<const uint4*>(&sb[buf][brw * kTileLd + kg * 8]));
     }
 #pragma unroll
     for (int am = 0; am < 4; ++am)
 #pragma unroll
-      for (int bn = 0; bn < 4; ++bn)
+      for (int bn = 0; bn < kOperands; ++bn)
         acc[am][bn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[bn], af[am], acc[am][bn], 0, 0, 0);
     if (more) stage(buf ^ 1);
     __syncthreads();
@@ -456,7 +466,16 @@ __global__ void __launch_bounds__(256)
     const int r = row0 + wm * 64 + am * 16 + i;
     if (r >= count) continue;
     const int pair = min(max(list[r], 0), n * top - 1);
-    if (GATED) {
+    if (GATED && SINGLE) {
+      bf16* dst = act_out + static_cast<size_t>(pair) * m;
+#pragma unroll
+      for (int bn = 0; bn < 4; ++bn) {
+        const int f = blockIdx.x * 128 + wn * 64 + bn * 16 + 4 * kg;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (f + q < m) dst[f + q] = from_float<bf16>(gate_act(acc[am][bn][q], act) * acc[am][bn][q]);
+      }
+    } else if (GATED) {
       bf16* dst = act_out + static_cast<size_t>(pair) * m;
 #pragma unroll
       for (int bn = 0; bn < 2; ++bn) {
@@ -579,9 +598,14 @@ extern "C" int shk_moe_experts_grouped(const void* x, const int32_t* chosen, con
   if (static_cast<long long>(n) * top >= 64LL * experts) {
     // lists of 64 pairs and more on average: tiles of 128 pairs through LDS
     const int row_tiles = (n + kTileRows - 1) / kTileRows;
-    moe_tiled_mfma_kernel<true><<<dim3((ff + 63) / 64, row_tiles, experts), 256, 0, s>>>(
-        static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
-        static_cast<bf16*>(act_buf), nullptr, n, width, ff, top, act);
+    if (w_gate == w_up)
+      moe_tiled_mfma_kernel<true, true><<<dim3((ff + 127) / 128, row_tiles, experts), 256, 0, s>>>(
+          static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
+          static_cast<bf16*>(act_buf), nullptr, n, width, ff, top, act);
+    else
+      moe_tiled_mfma_kernel<true><<<dim3((ff + 63) / 64, row_tiles, experts), 256, 0, s>>>(
+          static_cast<const bf16*>(x), order, counts, static_cast<const bf16*>(w_gate), static_cast<const bf16*>(w_up),
+          static_cast<bf16*>(act_buf), nullptr, n, width, ff, top, act);
     moe_tiled_mfma_kernel<false><<<dim3((width + 127) / 128, row_tiles, experts), 256, 0, s>>>(
         static_cast<const bf16*>(act_buf), order, counts, static_cast<const bf16*>(w_down), nullptr, nullptr, pair_out, n,
         ff, width, top, act);

@@ -9,6 +9,8 @@
 // activate_kernel        an activation of a plain product, elementwise
 // gate_mul_kernel        x * sigmoid(gate), elementwise
 // All arithmetic is float32.
+#include <initializer_list>
+
 #include "api.h"
 #include "common.h"
 
@@ -114,10 +116,33 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-template <typename T>
+// eight elements a thread in 16-byte pieces where the arrays allow it (V = 8), else one (V = 1)
+template <typename T, int V>
+__device__ __forceinline__ void load_run(const T* p, float (&x)[V]) {
+  if constexpr (V == 1) {
+    x[0] = to_float(p[0]);
+  } else {
+    const float4 a = ld4(p), b = ld4(p + 4);
+    x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+  }
+}
+template <typename T, int V>
+__device__ __forceinline__ void store_run(T* p, const float (&x)[V]) {
+  if constexpr (V == 1) {
+    p[0] = from_float<T>(x[0]);
+  } else {
+    st4(p, make_float4(x[0], x[1], x[2], x[3]));
+    st4(p + 4, make_float4(x[4], x[5], x[6], x[7]));
+  }
+}
+
+template <typename T, int V>
 __global__ void cast_rows_kernel(const float* __restrict__ src, T* __restrict__ dst, long long numel) {
-  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < numel) dst[i] = from_float<T>(src[i]);
+  const long long i = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) * V;
+  if (i >= numel) return;
+  float x[V];
+  load_run<float, V>(src + i, x);
+  store_run<T, V>(dst + i, x);
 }
 
 // 1: SiLU, 2: GELU (tanh form), 3: ReLU, 4: the square of ReLU
@@ -131,17 +156,35 @@ __device__ __forceinline__ float plain_act(float z, int act) {
   return z / (1.f + expf(-u));
 }
 
-template <typename T>
+template <typename T, int V>
 __global__ void activate_kernel(const T* __restrict__ x, T* __restrict__ out, long long numel, int act) {
-  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < numel) out[i] = from_float<T>(plain_act(to_float(x[i]), act));
+  const long long i = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) * V;
+  if (i >= numel) return;
+  float v[V];
+  load_run<T, V>(x + i, v);
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = plain_act(v[e], act);
+  store_run<T, V>(out + i, v);
 }
 
-template <typename T>
+template <typename T, int V>
 __global__ void gate_mul_kernel(const T* __restrict__ x, const T* __restrict__ gate, T* __restrict__ out,
                                 long long numel) {
-  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < numel) out[i] = from_float<T>(to_float(x[i]) / (1.f + expf(-to_float(gate[i]))));
+  const long long i = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) * V;
+  if (i >= numel) return;
+  float v[V], g[V];
+  load_run<T, V>(x + i, v);
+  load_run<T, V>(gate + i, g);
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = v[e] / (1.f + expf(-g[e]));
+  store_run<T, V>(out + i, v);
+}
+
+inline bool runs_of_eight(long long numel, std::initializer_list<const void*> arrays) {
+  if (numel % 8) return false;
+  for (const void* p : arrays)
+    if (reinterpret_cast<uintptr_t>(p) % 16) return false;
+  return true;
 }
 
 }  // namespace
@@ -191,11 +234,15 @@ extern "C" int shk_cast_rows(const float* src, void* dst, int dtype, long long n
   if (numel == 0) return 0;
   SHK_REQUIRE(src && dst, "cast_rows: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
-  if (dtype == kF32)
-    cast_rows_kernel<float><<<blocks, 256, 0, s>>>(src, static_cast<float*>(dst), numel);
-  else
-    cast_rows_kernel<bf16><<<blocks, 256, 0, s>>>(src, static_cast<bf16*>(dst), numel);
+#define SHK_GO(T, V) \
+  cast_rows_kernel<T, V><<<static_cast<unsigned>((numel / V + 255) / 256), 256, 0, s>>>(src, static_cast<T*>(dst), numel)
+  const bool eight = runs_of_eight(numel, {src, dst});
+  if (dtype == kF32) {
+    if (eight) SHK_GO(float, 8); else SHK_GO(float, 1);
+  } else {
+    if (eight) SHK_GO(bf16, 8); else SHK_GO(bf16, 1);
+  }
+#undef SHK_GO
   SHK_LAUNCH_CHECK("cast_rows");
   return 0;
 }
@@ -207,11 +254,16 @@ extern "C" int shk_activate(const void* x, void* out, int dtype, long long numel
   if (numel == 0) return 0;
   SHK_REQUIRE(x && out, "activate: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
-  if (dtype == kF32)
-    activate_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(x), static_cast<float*>(out), numel, act);
-  else
-    activate_kernel<bf16><<<blocks, 256, 0, s>>>(static_cast<const bf16*>(x), static_cast<bf16*>(out), numel, act);
+#define SHK_GO(T, V)                                                                                     \
+  activate_kernel<T, V><<<static_cast<unsigned>((numel / V + 255) / 256), 256, 0, s>>>(static_cast<const T*>(x), \
+                                                                                        static_cast<T*>(out), numel, act)
+  const bool eight = runs_of_eight(numel, {x, out});
+  if (dtype == kF32) {
+    if (eight) SHK_GO(float, 8); else SHK_GO(float, 1);
+  } else {
+    if (eight) SHK_GO(bf16, 8); else SHK_GO(bf16, 1);
+  }
+#undef SHK_GO
   SHK_LAUNCH_CHECK("activate");
   return 0;
 }
@@ -222,13 +274,16 @@ extern "C" int shk_gate_mul(const void* x, const void* gate, void* out, int dtyp
   if (numel == 0) return 0;
   SHK_REQUIRE(x && gate && out, "gate_mul: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
-  if (dtype == kF32)
-    gate_mul_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(x), static_cast<const float*>(gate),
-                                                  static_cast<float*>(out), numel);
-  else
-    gate_mul_kernel<bf16><<<blocks, 256, 0, s>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(gate),
-                                                 static_cast<bf16*>(out), numel);
+#define SHK_GO(T, V)                                                                                             \
+  gate_mul_kernel<T, V><<<static_cast<unsigned>((numel / V + 255) / 256), 256, 0, s>>>(                          \
+      static_cast<const T*>(x), static_cast<const T*>(gate), static_cast<T*>(out), numel)
+  const bool eight = runs_of_eight(numel, {x, gate, out});
+  if (dtype == kF32) {
+    if (eight) SHK_GO(float, 8); else SHK_GO(float, 1);
+  } else {
+    if (eight) SHK_GO(bf16, 8); else SHK_GO(bf16, 1);
+  }
+#undef SHK_GO
   SHK_LAUNCH_CHECK("gate_mul");
   return 0;
 }

@@ -91,6 +91,72 @@ __global__ void __launch_bounds__(kStoreThreads)
   }
 }
 
+// The same with normed queries and keys, a wavefront per head (of the queries, of the keys, of the
+// values): the head is held in registers between its mean square and its write, and a token's heads
+// spread over as many workgroups as it takes, so that a step of few tokens is not one long chain.
+constexpr int kMaxPerLane = 4;  // head sizes up to 256
+
+template <typename T>
+__global__ void __launch_bounds__(kStoreThreads)
+    qkv_norm_store_kernel(T* __restrict__ qkv, int heads, int kv_heads, int head_dim, int v_dim, float q_coef,
+                          int q_every, float v_eps, float qk_eps, const float* __restrict__ q_weight,
+                          const float* __restrict__ k_weight, int has_kv, const int32_t* __restrict__ positions,
+                          const int32_t* __restrict__ token_seq, const int32_t* __restrict__ tables,
+                          int table_stride, T* __restrict__ k_pool, T* __restrict__ v_pool, int page_size,
+                          int num_pages, int write_kv) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int unit = blockIdx.y * (kStoreThreads / kWave) + wave;
+  const int stored = (write_kv && has_kv) ? 2 * kv_heads : 0;
+  if (unit >= heads + stored) return;
+  const int pos = positions[t];
+  const int q_width = heads * head_dim, k_width = kv_heads * head_dim;
+  T* row = qkv + static_cast<size_t>(t) * (q_width + (has_kv ? k_width + kv_heads * v_dim : 0));
+  const bool is_q = unit < heads, is_k = !is_q && unit < heads + kv_heads;
+  const int g = is_q ? unit : is_k ? unit - heads : unit - heads - kv_heads;
+  const int size = (is_q || is_k) ? head_dim : v_dim;
+  T* src = row + (is_q ? g * head_dim : is_k ? q_width + g * head_dim : q_width + k_width + g * v_dim);
+  float x[kMaxPerLane];
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int d = lane + i * kWave;
+    x[i] = d < size ? to_float(src[d]) : 0.f;
+    sq = fmaf(x[i], x[i], sq);
+  }
+  const float eps = (is_q || is_k) ? qk_eps : v_eps;
+  float mult = eps > 0.f ? 1.f / sqrtf(wave_sum(sq) / static_cast<float>(size) + eps) : 1.f;
+  const float* weight = is_q ? q_weight : is_k ? k_weight : nullptr;
+  if (is_q) {
+    // 1 + coef * ln(floor((p + 1) / every) + 1), applied after the norm and its weight
+    const float factor = q_every > 0 ? 1.f + q_coef * logf(static_cast<float>((pos + 1) / q_every + 1)) : 1.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int d = lane + i * kWave;
+      if (d < size) src[d] = from_float<T>((weight ? x[i] * mult * weight[d] : x[i] * mult) * factor);
+    }
+    return;
+  }
+  int page = tables[static_cast<size_t>(token_seq[t]) * table_stride + pos / page_size];
+  if (page < 0 || page >= num_pages) return;  // a host bug; never dereferenced
+  const int slot = pos % page_size;
+  if (is_k) {
+    T* dst = k_pool + (static_cast<size_t>(page) * kv_heads + g) * page_size * head_dim;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int d = lane + i * kWave;
+      if (d < size) dst[key_offset(slot, d, page_size, head_dim)] = from_float<T>(weight ? x[i] * mult * weight[d] : x[i] * mult);
+    }
+  } else {
+    T* dst = v_pool + (static_cast<size_t>(page) * kv_heads + g) * v_dim * page_size + slot;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int d = lane + i * kWave;
+      if (d < size) dst[static_cast<size_t>(d) * page_size] = eps > 0.f ? from_float<T>(x[i] * mult) : src[d];
+    }
+  }
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -115,6 +181,23 @@ extern "C" int shk_qkv_store(void* qkv, int dtype, int n, int heads, int kv_head
                 "qkv_store: bad cache sizes page_size=%d num_pages=%d table_stride=%d", page_size, num_pages, table_stride);
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (qk_eps > 0.f && head_dim <= kMaxPerLane * kWave && v_dim <= kMaxPerLane * kWave) {
+    const int units = heads + ((write_kv && has_kv) ? 2 * kv_heads : 0);
+    const dim3 grid(n, (units + kStoreThreads / kWave - 1) / (kStoreThreads / kWave));
+    SHK_REQUIRE(grid.y <= 65535, "qkv_store: too many heads");
+    if (dtype == kF32)
+      qkv_norm_store_kernel<float><<<grid, kStoreThreads, 0, s>>>(
+          static_cast<float*>(qkv), heads, kv_heads, head_dim, v_dim, q_coef, q_every, v_eps, qk_eps, q_weight, k_weight,
+          has_kv, positions, token_seq, tables, table_stride, static_cast<float*>(k_pool), static_cast<float*>(v_pool),
+          page_size, num_pages, write_kv);
+    else
+      qkv_norm_store_kernel<bf16><<<grid, kStoreThreads, 0, s>>>(
+          static_cast<bf16*>(qkv), heads, kv_heads, head_dim, v_dim, q_coef, q_every, v_eps, qk_eps, q_weight, k_weight,
+          has_kv, positions, token_seq, tables, table_stride, static_cast<bf16*>(k_pool), static_cast<bf16*>(v_pool),
+          page_size, num_pages, write_kv);
+    SHK_LAUNCH_CHECK("qkv_store");
+    return 0;
+  }
   if (dtype == kF32)
     qkv_store_kernel<float><<<n, kStoreThreads, 0, s>>>(static_cast<float*>(qkv), heads, kv_heads, head_dim, v_dim,
                                                         q_coef, q_every, v_eps, qk_eps, q_weight, k_weight, has_kv,
