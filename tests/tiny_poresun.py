@@ -55,7 +55,7 @@ def _with(layer, mlp):
 
 
 POR_A = {
-    "architecture": "Poresun", "vocab": 211, "width": 70, "norm": {"eps": 1e-6}, "postln_alpha": 1.7,
+    "architecture": "Poresun", "vocab": 211, "width": 70, "norm": {"eps": 1e-6}, "postln_alpha": 1.2,
     "embedding": {"scale": 3.0},
     "layers": [
         _with(_attn("attention_2", 4, 2, 32, 16, 12, 40, temp=(0.4, 7)), _moe(5, 2, 24, shared=40)),
@@ -80,8 +80,8 @@ POR_B = {
 }
 
 POR_C = {
-    "architecture": "Poresun", "vocab": 300, "width": 128, "norm": {"eps": 2e-5}, "postln_alpha": 3.0,
-    "embedding": {"scale": 12.0},
+    "architecture": "Poresun", "vocab": 300, "width": 128, "norm": {"eps": 2e-5}, "postln_alpha": 1.6,
+    "embedding": {"scale": 4.0},
     "layers": [
         _with(_attn("attention", 8, 2, 64, 64, 32, 200, size=1000, cap=30.0, scale=0.2), _moe(8, 2, 48, shared=80)),
         _with(_attn("attention_2", 8, 1, 32, 32, 16, 64, temp=(0.5, 64)), _dense(256, 7.0)),
