@@ -519,7 +519,7 @@ def poresun_like(qcfg, window: int, pattern: str, experts: int, top: int):
     attention with weighted norms, a query temperature and the same table; s, such a layer
     that reads the keys and values of the last b layer before it; l, latent attention with as
     many heads, a query latent of 3/8 and a key/value latent of 1/8 of the width (rounded to
-    64), half a head rotated, and the output gate.  The first layer of every repetition has the
+    64, at most 512), half a head rotated, and the output gate.  The first layer of every repetition has the
     bounded gated feed-forward as wide as Qwen2's; the others `experts` routed experts without
     gates of which a token uses `top` (together half of Qwen2's feed-forward's multiply-adds)
     and a gated shared expert of the other half.  With it an object that names the sizes as the
@@ -535,8 +535,11 @@ def poresun_like(qcfg, window: int, pattern: str, experts: int, top: int):
     # an expert has two matrices where Qwen2's feed-forward has three
     ff = max(64, 3 * inter // (4 * top) // 64 * 64)
     shared = up64(3 * inter / 4)
-    latent = GatedLatentAttention(heads=H, dim=d, rot_dim=d // 2, vdim=d, q_rank=up64(3 * h / 8), kv_rank=up64(h / 8),
-                                  scale=(1.5 * d) ** -0.5, rot_base=10000.0, rot_dims=d // 2)
+    # (a key/value latent of at most 512: with the rotated part a cached row of at most 640 elements, which the
+    # latent attention's kernel on the matrix units takes)
+    latent = GatedLatentAttention(heads=H, dim=d, rot_dim=d // 2, vdim=d, q_rank=up64(3 * h / 8),
+                                  kv_rank=min(up64(h / 8), 512), scale=(1.5 * d) ** -0.5, rot_base=10000.0,
+                                  rot_dims=d // 2)
     layers, last_b = [], None
     for i in range(qcfg.num_hidden_layers):
         letter = pattern[i % len(pattern)]
