@@ -228,7 +228,7 @@ def test_configuration_reader_and_layout():
     assert [e.cache_of for e in spec.schedule] == [None, None, 0, None, 0]
     assert spec.blocks[2].mixer.shared_kv and not spec.blocks[0].mixer.shared_kv and spec.blocks[2].ffn is None
     assert spec.blocks[1].mixer.qk_norm == (1e-6, False) and spec.blocks[0].mixer.qk_norm == (1e-6, True)
-    assert spec.tie_word_embeddings and spec.embedding.scale == 3.0 and spec.blocks[3].alpha == 1.7
+    assert spec.tie_word_embeddings and spec.embedding.scale == 3.0 and spec.blocks[3].alpha == POR_A["postln_alpha"]
     _, model = _weights_for(POR_A)
     names = {p.name for p in model.params() if not p.optional}
     assert {"embed", "final.norm", "l0.mix.q.norm", "l0.mix.k.norm", "l0.mix.rel", "l0.ls1", "l0.ls2", "l1.mlp.gate",
