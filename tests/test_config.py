@@ -154,12 +154,14 @@ def test_default_model_dir_env_override(monkeypatch):
     import shrike_amd.models.ligipel as lg
     import shrike_amd.models.minilorn as n
     import shrike_amd.models.mofarax as m
+    import shrike_amd.models.poresun as po
     import shrike_amd.models.qwen2 as q
 
     importlib.reload(q)  # the reload emptied the registry; register again
     importlib.reload(m)
     importlib.reload(n)
     importlib.reload(lg)
+    importlib.reload(po)
 
 
 def test_plugins_named_in_the_environment_are_loaded_for_an_unknown_architecture(tmp_path, monkeypatch):
