@@ -112,7 +112,10 @@ int shk_interleave_gate_up(const void* gate_t, const void* up_t, int m, int k, v
 // bfloat16 row-major with row stride lda; out is bfloat16 or float32.
 // gated != 0: wt is an interleaved gate/up pair and out[n, m] = act(a @ gate^T) *
 // (a @ up^T), without bias or accumulation; gated is the activation, 1 for SiLU,
-// 2 for GELU in its tanh form.
+// 2 for GELU in its tanh form, 3 for ReLU, 4 for g * sigmoid(1.702 g).  A gated product's
+// `bias` is null or two floats, the gate's constants: with bias[0] > 0 the gate is bounded
+// from above and the other factor from both sides by it before anything else, and bias[1]
+// is added to that factor (as in shk_act_mul).
 // ksplit > 1 (at most 64 rows, float32 output, no bias): the k range is shared
 // by ksplit workgroups per block of weight rows and out is [ksplit][n][m], the
 // partial sums, which the kernel that reads the product adds up in order

@@ -67,13 +67,31 @@ __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); 
 // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) = g / (1 + exp(-2 u)).  Gated
 // kernels get the code in the argument that other products use for `accumulate`
 // (a gated product never accumulates).
-constexpr int kActSilu = 1, kActGeluTanh = 2;
+// kActRelu is max(g, 0), kActQuickGelu g / (1 + exp(-1.702 g)).
+constexpr int kActSilu = 1, kActGeluTanh = 2, kActRelu = 3, kActQuickGelu = 4;
 __device__ __forceinline__ float gate_act(float g, int act) {
   if (act == kActGeluTanh) {
     const float u = 0.7978845608028654f * (g + 0.044715f * g * g * g);
     return g / (1.f + __expf(-2.f * u));
   }
+  if (act == kActRelu) return fmaxf(g, 0.f);
+  if (act == kActQuickGelu) return g / (1.f + __expf(-1.702f * g));
   return silu(g);
+}
+
+// act(g) * u of a gated product.  A gate with constants brings them where other products bring their bias
+// (a gated product has none): args[0] > 0 bounds the gate from above and the other factor from both sides
+// before anything else, args[1] is added to that factor.
+__device__ __forceinline__ float gate_times_up(float g, float u, int act, const float* __restrict__ args) {
+  if (args) {
+    const float limit = args[0];
+    if (limit > 0.f) {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+    }
+    u += args[1];
+  }
+  return gate_act(g, act) * u;
 }
 
 template <int NB, int RB>
@@ -269,8 +287,8 @@ __global__ void __launch_bounds__(WAVES* kWave)
 #pragma unroll
       for (int w = 1; w < WAVES; ++w) up += red[w][RB - 1][b][ln][r];
     }
-    if (GATED) v = gate_act(v, accumulate) * up;
-    if (bias) v += bias[row];
+    if (GATED) v = gate_times_up(v, up, accumulate, bias);
+    if (!GATED && bias) v += bias[row];
     const size_t idx = static_cast<size_t>(token) * ldo + row;
     if (out_f32) {
       float* o = static_cast<float*>(out);
@@ -400,8 +418,8 @@ __global__ void __launch_bounds__(WAVES* kWave)
     float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      v[r] = GATED ? gate_act(acc[0][b][r], accumulate) * acc[RB - 1][b][r] : acc[0][b][r];
-      if (bias && row0 + r < m) v[r] += bias[row0 + r];
+      v[r] = GATED ? gate_times_up(acc[0][b][r], acc[RB - 1][b][r], accumulate, bias) : acc[0][b][r];
+      if (!GATED && bias && row0 + r < m) v[r] += bias[row0 + r];
     }
     if (ksplit > 1) {
       float* o = static_cast<float*>(out) + (static_cast<size_t>(blockIdx.y) * n + token) * ldo + row0;
@@ -465,7 +483,7 @@ __device__ __forceinline__ void big_store(const f32x4 (&acc)[WM][WN], int lane, 
       float v[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        v[r] = GATED ? gate_act(acc[i][jn][r], accumulate) * acc[i + (GATED ? 1 : 0)][jn][r]
+        v[r] = GATED ? gate_times_up(acc[i][jn][r], acc[i + (GATED ? 1 : 0)][jn][r], accumulate, bias)
                      : acc[i][jn][r] + add[GATED ? 0 : i][r];
       }
       const size_t idx = (static_cast<size_t>(share) * n + token) * ldo + row0;
@@ -1038,7 +1056,7 @@ __global__ void __launch_bounds__(16 * kWave)
         for (int b = 0; b < NB; ++b) {
           const f32x4 up = hand[((pair - first) * NB + b) * kWave + lane];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[b][r] = gate_act(acc[b][r], accumulate) * up[r];
+          for (int r = 0; r < 4; ++r) acc[b][r] = gate_times_up(acc[b][r], up[r], accumulate, bias);
         }
       }
     }
@@ -1057,7 +1075,7 @@ __global__ void __launch_bounds__(16 * kWave)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       v[r] = acc[b][r];
-      if (bias && row0 + r < m) v[r] += bias[row0 + r];
+      if (!GATED && bias && row0 + r < m) v[r] += bias[row0 + r];
     }
     if (ksplit > 1) {
       float* o = static_cast<float*>(out) + (static_cast<size_t>(blockIdx.y) * n + token) * ldo + row0;
@@ -1375,8 +1393,8 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
                                           void* out, int n, int m, int k, int lda, int ldo,
                                           int out_dtype, int accumulate, int gated, int ksplit,
                                           void* stream) {
-  SHK_REQUIRE(gated >= 0 && gated <= kActGeluTanh, "gemm_bf16: unknown gate activation %d", gated);
-  SHK_REQUIRE(!gated || (!accumulate && !bias), "gemm_bf16: a gated product takes no bias and does not accumulate");
+  SHK_REQUIRE(gated >= 0 && gated <= kActQuickGelu, "gemm_bf16: unknown gate activation %d", gated);
+  SHK_REQUIRE(!gated || !accumulate, "gemm_bf16: a gated product does not accumulate");
   SHK_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_bf16: ksplit %d is outside 1..64", ksplit);
   SHK_REQUIRE(ksplit == 1 || (!gated && !accumulate && !bias && out_dtype == kF32 && ldo == m),
               "gemm_bf16: a product split along k writes plain float32 partial sums [ksplit][n][m]");
@@ -1409,7 +1427,8 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
       launch_big<4, 4, 4, 4, 1>(s, ap, lda, n, k, wp, kt, main_rows, bias, out, ldo, of, accumulate,
                                 vec, gated, main_blocks, 1);
       const uint4* rest_w = wp + static_cast<size_t>(main_blocks) * kt * kWave;
-      const float* rest_bias = bias ? bias + main_rows : nullptr;
+      // (a gated product's `bias` is its gate's two constants, the same for every row)
+      const float* rest_bias = (bias && !gated) ? bias + main_rows : bias;
       void* rest_out = of ? static_cast<void*>(static_cast<float*>(out) + main_rows)
                           : static_cast<void*>(static_cast<bf16*>(out) + main_rows);
       if (rest_shape == 0)

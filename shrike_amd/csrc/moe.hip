@@ -260,6 +260,36 @@ __global__ void __launch_bounds__(256)
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b) accg[a][b] = accu[a][b] = mf32x4{0.f, 0.f, 0.f, 0.f};
+  if (single) {
+    // one matrix: four steps' operands are asked for at once (eight 16-byte pieces of weights a lane in
+    // flight: few wavefronts run, and what they have in flight is what the memory delivers); the sums
+    // still run over k in ascending order
+    constexpr int kAhead = 4;
+    for (int k0 = 0; k0 < width; k0 += 32 * kAhead) {
+      uint4 av[kAhead][2], gv[kAhead][2];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int kk = k0 + 32 * u;
+        const bool have = kk + kg * 8 < width;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          av[u][a] = gv[u][a] = make_uint4(0, 0, 0, 0);
+          if (have) {
+            gv[u][a] = *reinterpret_cast<const uint4*>(gr[a] + kk);
+            if (pair[a] >= 0) av[u][a] = *reinterpret_cast<const uint4*>(xr[a] + kk);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u)
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+            accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, gv[u][b]),
+                                                                 __builtin_bit_cast(mbf16x8, av[u][a]), accg[a][b], 0, 0, 0);
+    }
+  } else {
   for (int k0 = 0; k0 < width; k0 += 32) {
     const bool have = k0 + kg * 8 < width;  // (width is a multiple of 8: a piece is whole or absent)
     uint4 av[2], gv[2], uv[2];
@@ -269,7 +299,7 @@ __global__ void __launch_bounds__(256)
       if (have) {
         if (pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(xr[a] + k0);
         gv[a] = *reinterpret_cast<const uint4*>(gr[a] + k0);
-        if (!single) uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
+        uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
       }
     }
 #pragma unroll
@@ -278,10 +308,10 @@ __global__ void __launch_bounds__(256)
       for (int b = 0; b < 2; ++b) {
         accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, gv[b]),
                                                              __builtin_bit_cast(mbf16x8, av[a]), accg[a][b], 0, 0, 0);
-        if (!single)
-          accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
-                                                               __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
+        accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
+                                                             __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
       }
+  }
   }
   // features were the rows of the products: this lane holds features f0 + 16 b + 4 kg + r of pair row a * 16 + i
 #pragma unroll
@@ -331,25 +361,34 @@ __global__ void __launch_bounds__(256)
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = mf32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < ff; k0 += 32) {
-    const bool have = k0 + kg * 8 < ff;
-    uint4 av[2], wv[4];
+  // two steps' operands are asked for at once (eight 16-byte pieces of weights a lane in flight); the sums
+  // run over k in ascending order all the same
+  constexpr int kAhead = 2;
+  for (int k0 = 0; k0 < ff; k0 += 32 * kAhead) {
+    uint4 av[kAhead][2], wv[kAhead][4];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      av[a] = make_uint4(0, 0, 0, 0);
-      if (have && pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(ar[a] + k0);
+    for (int u = 0; u < kAhead; ++u) {
+      const int kk = k0 + 32 * u;
+      const bool have = kk + kg * 8 < ff;
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        av[u][a] = make_uint4(0, 0, 0, 0);
+        if (have && pair[a] >= 0) av[u][a] = *reinterpret_cast<const uint4*>(ar[a] + kk);
+      }
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        wv[u][b] = make_uint4(0, 0, 0, 0);
+        if (have) wv[u][b] = *reinterpret_cast<const uint4*>(wr[b] + kk);
+      }
     }
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      wv[b] = make_uint4(0, 0, 0, 0);
-      if (have) wv[b] = *reinterpret_cast<const uint4*>(wr[b] + k0);
-    }
+    for (int u = 0; u < kAhead; ++u)
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < 2; ++a)
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
-        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, wv[b]),
-                                                            __builtin_bit_cast(mbf16x8, av[a]), acc[a][b], 0, 0, 0);
+        for (int b = 0; b < 4; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, wv[u][b]),
+                                                              __builtin_bit_cast(mbf16x8, av[u][a]), acc[a][b], 0, 0, 0);
   }
 #pragma unroll
   for (int a = 0; a < 2; ++a) {

@@ -18,12 +18,13 @@ from ..kernels import ops
 class LinearWeight:
     """A weight matrix [rows, cols] as the kernels want it."""
 
-    __slots__ = ("rows", "cols", "dense", "tiled")
+    __slots__ = ("rows", "cols", "dense", "tiled", "gate_args")
 
-    def __init__(self, shape, dense: torch.Tensor | None, tiled: torch.Tensor | None):
+    def __init__(self, shape, dense: torch.Tensor | None, tiled: torch.Tensor | None, gate_args=None):
         self.rows, self.cols = shape
         self.dense = dense  # row-major (float32 path)
         self.tiled = tiled  # MFMA operand layout (bfloat16 path)
+        self.gate_args = gate_args  # (limit, up_shift) on the device, for a gate with constants
 
 
 class Runtime:
@@ -40,26 +41,26 @@ class Runtime:
             return LinearWeight(w.shape, None, ops.retile_weight(w))
         return LinearWeight(w.shape, w, None)
 
-    @staticmethod
-    def fused_gate(activation: str = "silu", limit=None, up_shift: float = 0.0) -> bool:
-        """Whether the bfloat16 product's epilogue applies this gate itself."""
-        return activation in ("silu", "gelu_tanh") and limit is None and up_shift == 0.0
-
     def gated_weight(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu", limit=None,
                      up_shift: float = 0.0):
-        """The two matrices of a gated feed-forward, as `gated_linear` wants them for this gate."""
-        if self.dtype == torch.bfloat16 and self.fused_gate(activation, limit, up_shift):
+        """The two matrices of a gated feed-forward, as `gated_linear` wants them for this gate
+        (bfloat16: interleaved tiles for the product whose epilogue applies the gate, and the
+        gate's constants on the device where it has any)."""
+        if self.dtype == torch.bfloat16:
             tiled = ops.interleave_gate_up(gate.contiguous(), up.contiguous())
-            return LinearWeight(gate.shape, None, tiled)
+            args = None
+            if limit is not None or up_shift != 0.0:
+                args = torch.tensor([float(limit or 0.0), float(up_shift)], dtype=torch.float32, device=self.device)
+            return LinearWeight(gate.shape, None, tiled, args)
         return self.weight(torch.cat([gate, up], dim=0))
 
     def gated_linear(self, ctx, x, w: LinearWeight, out, activation: str = "silu", limit=None,
                      up_shift: float = 0.0) -> None:
         """out = act(g) * (u + up_shift), g = x @ gate.T, u = x @ up.T, both bounded by `limit` first
-        where one is given.  bfloat16 with a gate that the product's epilogue applies: one product;
-        else product, then activation."""
-        if w.tiled is not None and self.fused_gate(activation, limit, up_shift):
-            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, gated=activation)
+        where one is given.  bfloat16: one product whose epilogue applies the gate (its constants are
+        those the weight was made with); float32: product, then activation."""
+        if w.tiled is not None:
+            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, gated=activation, gate_args=w.gate_args)
             return
         gate_up = ctx.buffer("ffn_gate_up", (x.shape[0], w.rows), self.dtype)
         self.linear(x, w, gate_up)

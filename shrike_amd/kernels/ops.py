@@ -395,13 +395,14 @@ def mfma_alone(operands: torch.Tensor, workgroups: int, iters: int) -> float:
 
 
 def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, gated=False,
-                      splits: int = 1) -> None:
+                      splits: int = 1, gate_args=None) -> None:
     """out (+)= a @ w.T + bias with wt = retile_weight(w): up to 64 rows of a
     stream the weights once; more rows run the LDS-staged MFMA kernel (tiles of
     128 x 128 to 256 x 256, chosen by how many the product has).
     splits > 1: out is float32 [splits, n, m] and receives partial sums.
-    gated: False, or the gate's activation ("silu", "gelu_tanh"; True is "silu") for
-    an interleaved gate/up weight."""
+    gated: False, or the gate's activation (one of GATE_ACTIVATIONS; True is "silu") for
+    an interleaved gate/up weight.  gate_args: float32 [2] on the device, (limit, up_shift) of
+    such a gate: act(min(g, limit)) * (clamp(u, -limit, limit) + up_shift), limit 0: no bounds."""
     _rows(a, "gemm a")
     n = a.shape[0]
     if a.shape[1] != k or a.dtype != torch.bfloat16:
@@ -417,6 +418,10 @@ def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, g
         raise KernelError("gemm_tiled_weight: wt is not the tiled layout of an [m, k] matrix")
     if bias is not None and bias.numel() != m:
         raise KernelError(f"gemm_tiled_weight: bias has {bias.numel()} elements, m is {m}")
+    if gate_args is not None:
+        if not gated or bias is not None or gate_args.numel() != 2 or gate_args.dtype != torch.float32:
+            raise KernelError("gemm_tiled_weight: gate_args are two float32 numbers of a gated product without bias")
+        bias = gate_args  # (they travel in the bias's place)
     check(
         load().shk_gemm_bf16_tiled_weight(
             _dev(a, "a"), _dev(wt, "wt"),

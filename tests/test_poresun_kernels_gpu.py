@@ -134,6 +134,28 @@ def test_gate_with_a_limit(ops, dtype, limit, shift):
         close(out, plain.dense_ff(x, w, "p", {"limit": limit}), dtype)
 
 
+@pytest.mark.parametrize("n", [1, 8, 40, 64, 300, 2100])
+@pytest.mark.parametrize("limit, shift, activation", [(1.0, 1.0, "quick_gelu"), (None, 1.0, "quick_gelu"), (3.0, 0.0, "silu"),
+                                                      (None, 0.0, "relu")])
+def test_gated_product_applies_a_gate_with_constants(ops, n, limit, shift, activation):
+    """The bfloat16 gate/up product whose epilogue bounds, activates, shifts and multiplies, in each
+    of its kernels (few tokens, some dozens, hundreds, thousands), against product-then-activation."""
+    torch.manual_seed(11)
+    k, ff = 96, 200
+    x = (torch.randn(n, k) * 2).to(torch.bfloat16)
+    gate, up = (torch.randn(ff, k) * 0.3).to(torch.bfloat16), (torch.randn(ff, k) * 0.3).to(torch.bfloat16)
+    wt = ops.interleave_gate_up(dev(gate), dev(up))
+    args = None if limit is None and shift == 0.0 else torch.tensor([limit or 0.0, shift], device="cuda")
+    out = torch.empty(n, ff, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_tiled_weight(dev(x), wt, ff, k, out, gated=activation, gate_args=args)
+    g, u = x.double() @ gate.double().T, x.double() @ up.double().T
+    if limit:
+        assert float(g.max()) > limit and float(u.min()) < -limit
+        g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+    act = {"quick_gelu": lambda z: z * torch.sigmoid(1.702 * z), "silu": lambda z: z * torch.sigmoid(z), "relu": torch.relu}[activation]
+    close(out, act(g) * (u + shift), torch.bfloat16)
+
+
 # ------------------------------------------------------------------ cache write with normed queries and keys
 
 @pytest.mark.parametrize("dtype", DTYPES)
