@@ -153,7 +153,12 @@ class PagedAttention(Mixer):
     (reference: shrike/models/qwen.py:111-125, shrike/engine/model_runner.py:63-151).
     Beyond the reference's model, by the spec: a window, a block-local mask
     (`chunk`), and values that are the keys before their rotation
-    (`values_from_keys`: no value projection, the cache still holds both).
+    (`values_from_keys`: no value projection, the cache still holds both);
+    without rotation also values of another size than keys, a query temperature,
+    normed values, normed queries and keys (with or without weights), capped
+    scores, sinks, a learned bias by distance from a table (laid out by distance
+    when the weights are loaded), and layers without keys and values of their
+    own that read another run's cache.
 
     The three projections are stacked into one [(H + 2 Hkv) D, h] matrix at
     load time; head j of q is rows j*D..(j+1)*D-1 of the q part, as in the

@@ -253,3 +253,33 @@ def test_configuration_reader_and_layout():
     ):
         with pytest.raises(ConfigError, match=text):
             arch.config_cls.from_dict(broken)
+
+
+def test_a_bias_tables_rows_are_the_files_own(tmp_path):
+    """config.json need not count the bias table's rows: the tensor's shape gives them, the loader
+    accepts any count for that size alone, and the engine's table by distance follows the file."""
+    import json
+
+    from shrike_amd.config.registry import load_model_config
+    from shrike_amd.models import DecoderModel
+    from shrike_amd.weights import write_model_folder
+    from shrike_amd.weights.loader import WeightError, _index, check_names, shard_files
+
+    folder = write_model_folder(dict(POR_A), tmp_path / "m", seed=3, dtype="float32")
+    cfg = json.loads((folder / "config.json").read_text())
+    for layer in cfg["layers"]:
+        layer["mixer"].pop("bias_rows", None)
+    (folder / "config.json").write_text(json.dumps(cfg))
+    _, spec = load_model_config(folder)
+    assert spec.blocks[0].mixer.bucket_bias == (None, 40)
+    params = DecoderModel(spec).params()
+    rel = next(p for p in params if p.name == "l0.mix.rel")
+    assert rel.shape == (None, 4) and rel.drawn_shape() == (32, 4) and rel.matches((12, 4)) and not rel.matches((12, 5))
+    check_names(_index(shard_files(folder)), params)  # 12, 7, 20 and 2 rows: all taken as they are
+    # the plain form reads the same folder
+    logits = P.PlainPoresun(folder).logits([1, 2, 3, 4, 5, 6, 7, 8, 9])
+    assert torch.isfinite(logits).all()
+    # another size of the same tensor is still an error
+    wrong = [p if p.name != "l0.mix.rel" else type(p)(p.name, (None, 5), p.init, p.keep_float32) for p in params]
+    with pytest.raises(WeightError, match="l0.mix.rel"):
+        check_names(_index(shard_files(folder)), wrong)
