@@ -28,12 +28,12 @@ def test_buckets_by_hand():
     # an odd count: half is 3, four rows for the logarithm
     assert [P.distance_bucket(d, 7, 30) for d in (2, 3, 5, 6, 10, 11, 17, 29, 30)] == [2, 3, 3, 4, 5, 5, 6, 6, 6]
     # rows never fall as the distance grows, and the last one is reached at `reach` at the latest
-    for rows, reach in ((2, 3), (16, 64), (32, 240), (40, 500), (9, 25)):
+    for rows, reach in ((2, 3), (16, 64), (24, 300), (40, 500), (9, 25)):
         seq = [P.distance_bucket(d, rows, reach) for d in range(reach + 5)]
         assert seq == sorted(seq) and seq[reach] == rows - 1 and seq[0] == 0
 
 
-@pytest.mark.parametrize("rows, reach", [(2, 3), (7, 30), (12, 40), (16, 120), (32, 240), (40, 500), (9, 25)])
+@pytest.mark.parametrize("rows, reach", [(2, 3), (7, 30), (12, 40), (14, 90), (24, 300), (40, 500), (9, 25)])
 def test_the_engines_table_of_buckets_is_the_plain_one(rows, reach):
     from shrike_amd.parts.attention import distance_buckets
 

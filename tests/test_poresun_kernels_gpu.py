@@ -160,7 +160,7 @@ def test_gated_product_applies_a_gate_with_constants(ops, n, limit, shift, activ
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim, page_size, weighted, every",
-                         [(6, 2, 40, 72, 16, True, 100), (3, 3, 8, 5, 4, False, 0), (8, 1, 64, 64, 8, True, 1),
+                         [(6, 2, 40, 72, 16, True, 100), (3, 3, 8, 5, 4, False, 0), (10, 2, 64, 64, 8, True, 1),
                           (2, 2, 128, 32, 16, False, 3)])
 def test_cache_write_with_normed_queries_and_keys(ops, dtype, heads, kv_heads, dim, vdim, page_size, weighted, every):
     torch.manual_seed(7)
@@ -265,8 +265,8 @@ CASES = [
     (6, 2, 40, 72, 16, None, 45.0, 12, 40),
     (3, 3, 32, 32, 8, 37, 4.0, 7, 30),
     (6, 1, 24, 7, 4, 1, None, 2, 3),
-    (8, 1, 64, 64, 16, 72, 20.0, 16, 120),
-    (8, 2, 64, 64, 16, None, None, 32, 240),
+    (10, 2, 64, 64, 16, 50, 12.0, 14, 90),
+    (6, 2, 64, 64, 16, None, None, 24, 300),
     (4, 4, 128, 128, 32, 300, 30.0, 40, 500),
     (16, 1, 32, 32, 16, 16, 9.0, 9, 25),
 ]

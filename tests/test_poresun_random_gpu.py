@@ -76,8 +76,8 @@ def draw_config(seed: int) -> dict:
         layer = rng.choice([draw_attention, draw_attention, draw_latent])(rng, i, owners)
         layers.append({**layer, "mlp": draw_mlp(rng)})
     return {"architecture": "Poresun", "vocab": rng.choice([61, 97, 700, 3000]), "width": rng.choice([40, 72, 128, 200, 320]),
-            "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])}, "postln_alpha": rng.choice([0.7, 1.0, 1.5, 2.5, 4.0]),
-            "embedding": {"scale": rng.choice([0.5, 1.0, 3.0, 12.0])}, "layers": layers}
+            "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])}, "postln_alpha": rng.choice([0.7, 1.0, 1.5, 2.0, 4.0]),
+            "embedding": {"scale": rng.choice([0.5, 1.0, 3.0, 9.0])}, "layers": layers}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

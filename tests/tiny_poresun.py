@@ -84,7 +84,7 @@ POR_C = {
     "embedding": {"scale": 4.0},
     "layers": [
         _with(_attn("attention", 8, 2, 64, 64, 32, 200, size=1000, cap=30.0, scale=0.2), _moe(8, 2, 48, shared=80)),
-        _with(_attn("attention_2", 8, 1, 32, 32, 16, 64, temp=(0.5, 64)), _dense(256, 7.0)),
+        _with(_attn("attention_2", 8, 1, 32, 32, 18, 64, temp=(0.3, 64)), _dense(256, 7.0)),
         _with(_latent(4, 32, 32, 64, 64, 96, base=1.0e5), _moe(8, 8, 32, shared=32)),
         _with(_attn("attention", 4, 4, 32, 32, 8, 20, size=16, cap=15.0), _moe(4, 1, 128)),
     ],
