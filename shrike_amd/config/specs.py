@@ -347,7 +347,9 @@ class PostNormBlockSpec:
     x <- mixer_norm(alpha * x + s1 * mixer(x)); x <- ffn_norm(alpha * x + s2 * ffn(x)), the
     sublayers reading x itself.  ``layer_scale``: s1 and s2 are learned vectors of the model's
     width (tensors ``mixer_scale_name`` / ``ffn_scale_name`` below the block's name); else ones.
-    ``ffn`` may be None: the layer then has no feed-forward, no second norm and no second scale."""
+    ``ffn`` may be None: the layer then has no feed-forward and no second scale; it has a second
+    norm only if ``ffn_norm`` is given and the weight file holds its tensor, and the stream then
+    passes it with nothing added, x <- ffn_norm(alpha * x)."""
 
     kind: ClassVar[str] = "postnorm_residual"
     name: str

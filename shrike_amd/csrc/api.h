@@ -80,8 +80,8 @@ int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act,
 
 // A stream that is normed after every sum (postnorm.hip): resid[r, :] <- (x / sqrt(mean(x^2) + eps)) *
 // weight with x = alpha * resid[r, :] + lscale * delta[r, :] (lscale float32 [hidden] or null: ones);
-// delta has `dtype`, or is float32 partial sums [delta_splits][n][hidden] added in order.  cast (of
-// `dtype`, or null) receives the new rows too.
+// delta has `dtype`, or is float32 partial sums [delta_splits][n][hidden] added in order, or is null
+// (nothing is added).  cast (of `dtype`, or null) receives the new rows too.
 int shk_postnorm(float* resid, const void* delta, int delta_splits, float alpha, const float* lscale,
                  const float* weight, float eps, void* cast, int dtype, int n, int hidden, void* stream);
 // dst[i] = src[i] in `dtype`.

@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(THREADS)
   __shared__ float scratch[16];
   const size_t row = blockIdx.x;
   float* x = resid + row * hidden;
-  const TD* d = delta + row * hidden;
+  const TD* d = delta ? delta + row * hidden : nullptr;  // (null: nothing is added)
   const int nvec = hidden / 4;
   float4 v[kPostVecs], dv[kPostVecs], w[kPostVecs], ls[kPostVecs];
 #pragma unroll
@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(THREADS)
     ls[i] = make_float4(1.f, 1.f, 1.f, 1.f);
     if (c < nvec) {
       v[i] = ld4(x + c * 4);
-      dv[i] = ld4(d + c * 4);
+      if (d) dv[i] = ld4(d + c * 4);
       w[i] = ld4(weight + c * 4);
       if (lscale) ls[i] = ld4(lscale + c * 4);
     }
@@ -98,10 +98,10 @@ __global__ void __launch_bounds__(256)
   __shared__ float scratch[16];
   const size_t row = blockIdx.x;
   float* x = resid + row * hidden;
-  const TD* d = delta + row * hidden;
+  const TD* d = delta ? delta + row * hidden : nullptr;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += 256) {
-    float add = to_float(d[i]);
+    float add = d ? to_float(d[i]) : 0.f;
     for (int z = 1; z < splits; ++z) add += to_float(d[z * split_stride + i]);
     const float v = fmaf(alpha, x[i], (lscale ? lscale[i] : 1.f) * add);
     sums[i] = v;
@@ -200,7 +200,7 @@ extern "C" int shk_postnorm(float* resid, const void* delta, int delta_splits, f
               delta_splits);
   SHK_REQUIRE(hidden <= 15000, "postnorm: rows of %d elements do not fit a workgroup's LDS", hidden);
   if (n == 0) return 0;
-  SHK_REQUIRE(resid && delta && weight, "postnorm: null pointer");
+  SHK_REQUIRE(resid && weight && (delta || delta_splits == 0), "postnorm: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t stride = static_cast<size_t>(n) * hidden;
   const bool vec = hidden % 4 == 0 && hidden <= 8192;

@@ -275,8 +275,8 @@ def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu", 
 
 def postnorm(resid, delta, alpha: float, lscale, weight, eps: float, cast=None, dtype=None) -> None:
     """resid <- rmsnorm(alpha * resid + lscale * delta) * weight, row by row in float32 (lscale float32
-    [hidden] or None: ones; delta a tensor of the compute dtype or a SplitSum); `cast`, if given,
-    receives the new rows in the compute dtype."""
+    [hidden] or None: ones; delta a tensor of the compute dtype, a SplitSum, or None: nothing is
+    added); `cast`, if given, receives the new rows in the compute dtype."""
     n, hidden = resid.shape
     dtype = cast.dtype if cast is not None else dtype
     if dtype is None:
@@ -285,7 +285,7 @@ def postnorm(resid, delta, alpha: float, lscale, weight, eps: float, cast=None, 
         raise KernelError("postnorm: resid and cast must be contiguous and of one shape")
     if weight.numel() != hidden or (lscale is not None and lscale.numel() != hidden):
         raise KernelError(f"postnorm: weight and lscale must have {hidden} elements")
-    p, splits = _delta(delta, resid, dtype, "postnorm")
+    p, splits = (None, 0) if delta is None else _delta(delta, resid, dtype, "postnorm")
     check(load().shk_postnorm(_dev(resid, "resid", torch.float32), p, splits, float(alpha),
                               None if lscale is None else _dev(lscale, "lscale", torch.float32),
                               _dev(weight, "weight", torch.float32), float(eps),

@@ -361,8 +361,7 @@ def build_spec(cfg: PoresunConfig) -> ModelSpec:
         own = layer.type != "latent_attention" and layer.mixer.kv_from is None
         window = kept[i] if own and kept[i] != layer.mixer.window else "own"
         blocks.append(PostNormBlockSpec(name=f"l{i}", mixer=mixer_spec(layer, cfg.norm_eps, window),
-                                        ffn=ffn_spec(layer.mlp), mixer_norm=norm,
-                                        ffn_norm=norm if layer.mlp is not None else None, alpha=cfg.alpha,
+                                        ffn=ffn_spec(layer.mlp), mixer_norm=norm, ffn_norm=norm, alpha=cfg.alpha,
                                         layer_scale=True))
         schedule.append(ScheduleEntry(i, cache_of=getattr(layer.mixer, "kv_from", None)))
     return ModelSpec(

@@ -167,7 +167,9 @@ class PostNormResidualBlock(Block):
     after the sum, the stream is what the norm leaves, and the sublayers read the stream itself.
     One kernel per sublayer forms the scaled sum in float32 (adding up the parts of a split
     product in order), norms it, stores it as the float32 stream and leaves it in the compute
-    dtype for the products that read it next."""
+    dtype for the products that read it next.  A layer without a feed-forward has no second norm
+    unless its spec names one and the weight file holds that norm's tensor: then the stream
+    passes it with nothing added, x <- norm2(alpha x)."""
 
     def __init__(self, spec, width, name):
         super().__init__(spec, width, name)
@@ -176,6 +178,7 @@ class PostNormResidualBlock(Block):
         self.ffn = self.ffn_norm = None
         if spec.ffn is not None:
             self.ffn = build_part("ffn", spec.ffn, width, f"{name}.{spec.ffn_name}")
+        if spec.ffn is not None or spec.ffn_norm is not None:
             self.ffn_norm = build_part("norm", spec.ffn_norm, width, f"{name}.{spec.ffn_norm_name}")
         self.parts = tuple(p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None)
         self.parts += tuple(getattr(self.mixer, "parts", ()))
@@ -188,13 +191,21 @@ class PostNormResidualBlock(Block):
         s = self.spec
         if not s.layer_scale:
             return ()
-        return (f"{self.name}.{s.mixer_scale_name}",) + ((f"{self.name}.{s.ffn_scale_name}",) if self.ffn else ())
+        return (f"{self.name}.{s.mixer_scale_name}",) + ((f"{self.name}.{s.ffn_scale_name}",) if self.ffn_norm else ())
 
     def params(self):
+        from dataclasses import replace
+
         from .base import ParamSpec
 
-        out = [p for part in self._own() for p in part.params()]
-        return out + [ParamSpec(n, (self.width,), init="norm", keep_float32=True) for n in self._scale_names()]
+        out = []
+        for part in self._own():
+            # the second norm of a layer without a feed-forward: there only if the file has it
+            loose = part is self.ffn_norm and self.ffn is None
+            out += [replace(p, optional=True) if loose else p for p in part.params()]
+        for i, n in enumerate(self._scale_names()):
+            out.append(ParamSpec(n, (self.width,), init="norm", keep_float32=True, optional=i == 1 and self.ffn is None))
+        return out
 
     def check(self, runtime):
         for part in (self.mixer_norm, self.ffn_norm):
@@ -212,12 +223,14 @@ class PostNormResidualBlock(Block):
         return all(part.launches_follow_shape for part in self.parts)
 
     def load(self, tensors, runtime):
+        if self.ffn is None and self.ffn_norm is not None and any(p.name not in tensors for p in self.ffn_norm.params()):
+            self.ffn_norm = None  # the file has no second norm for this layer: the stream does not pass one
         for part in self._own():
             part.load(tensors, runtime)
         names = self._scale_names()
         if names:
             self.mixer_scale = tensors[names[0]].contiguous()
-            self.ffn_scale = tensors[names[1]].contiguous() if self.ffn else None
+            self.ffn_scale = tensors[names[1]].contiguous() if self.ffn is not None else None
         self.alpha = float(self.spec.alpha)
 
     def forward(self, ctx, hidden: HiddenState, cache) -> None:
@@ -235,9 +248,10 @@ class PostNormResidualBlock(Block):
         mixed = self.mixer.forward(ctx, x, cache)
         ops.postnorm(hidden.resid, mixed, self.alpha, self.mixer_scale, self.mixer_norm.weight, self.mixer_norm.eps,
                      cast=out, dtype=ctx.dtype)
-        if self.ffn is not None:
-            x = hidden.resid if in_float32 else out
-            fed = self.ffn.forward(ctx, x)
+        if self.ffn_norm is not None:
+            fed = None
+            if self.ffn is not None:
+                fed = self.ffn.forward(ctx, hidden.resid if in_float32 else out)
             ops.postnorm(hidden.resid, fed, self.alpha, self.ffn_scale, self.ffn_norm.weight, self.ffn_norm.eps,
                          cast=out, dtype=ctx.dtype)
         hidden.cast = out

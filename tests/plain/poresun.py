@@ -217,6 +217,8 @@ def forward(cfg: dict, w: dict, tokens, return_layers: bool = False):
         x = normed_sum(x, y, w[p + ".ls1"], alpha, w[p + ".norm1"], eps)
         if layer.get("mlp"):
             x = normed_sum(x, feed_forward(x, w, p + ".mlp", layer["mlp"]), w[p + ".ls2"], alpha, w[p + ".norm2"], eps)
+        elif p + ".norm2" in w:  # a file that holds a second norm for a layer without a feed-forward
+            x = normed_sum(x, torch.zeros_like(x), 1.0, alpha, w[p + ".norm2"], eps)
         streams.append(x)
     logits = (unit_rms(x, eps) * w["final.norm"]) @ w["embed"].T
     return (logits, torch.stack(streams)) if return_layers else logits

@@ -252,6 +252,40 @@ def test_graphs_and_recorded_launches_equal_kernel_by_kernel_steps(name, dtype, 
     assert torch.equal(results[0], results[1])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_without_feed_forward_passes_a_second_norm_if_the_file_holds_one(dtype, model_root, tmp_path):
+    """The same tiny model with one more tensor, a second norm for its layer without a feed-forward:
+    the stream passes it with nothing added, x <- norm2(alpha x); without the tensor it does not."""
+    import json
+    import shutil
+
+    from safetensors.torch import load_file, save_file
+    from shrike_amd.engine.runner import StepEntry
+
+    src = make_model_dir("A", model_root, dtype=dtype)
+    folder = tmp_path / "with_norm2"
+    shutil.copytree(src, folder)
+    tensors = load_file(str(folder / "model.safetensors"))
+    assert "l2.norm2" not in tensors and json.loads((folder / "config.json").read_text())["layers"][2]["mlp"] is None
+    tensors["l2.norm2"] = (1.0 + 0.3 * torch.randn(tensors["l2.norm1"].shape)).to(tensors["l2.norm1"].dtype)
+    save_file(tensors, str(folder / "model.safetensors"))
+    ids = requests_for("A", [60])["r0"]
+    results = {}
+    for name, path in (("without", src), ("with", folder)):
+        want = PlainPoresun(path).logits(ids)
+        model, cache, runner = engine_parts(path, dtype, 16, 16)
+        seq = cache.new_sequence()
+        cache.append(seq, 0, len(ids))
+        got = runner.step([StepEntry(seq, ids, 0, list(range(len(ids))))]).cpu().double()
+        err = (got - want).abs().amax(-1) / want.abs().max()
+        if dtype == "float32":
+            assert float(err.max()) <= TOL[dtype], f"{name}: rel err {float(err.max()):.3e}"
+        else:
+            assert float((err > TOL[dtype]).float().mean()) <= 0.06, f"{name}: {int((err > TOL[dtype]).sum())} rows over"
+        results[name] = want
+    assert float((results["with"] - results["without"]).abs().max()) > 1e-2 * float(results["with"].abs().max())
+
+
 def test_command_line_generates_with_a_model_folder(model_root, capsys):
     from shrike_amd.__main__ import main
 
