@@ -281,7 +281,8 @@ def test_attention_with_a_bias_table(ops, dtype, heads, kv_heads, dim, vdim, pag
     700 keys.  For every sequence's last query one key is made to stand out (a score of 12
     before the cap): far back where there is no window, else the oldest key inside the window, and
     the query before it points as strongly at the first key behind its own window (which must not
-    show).  The table's entries
+    show); the key just behind the last query's window, single tokens included, is a stronger copy of
+    the one it may see.  The table's entries
     are several units apart, so that a wrong row shows too."""
     from shrike_amd.parts.attention import distance_buckets
 
@@ -302,6 +303,10 @@ def test_attention_with_a_bias_table(ops, dtype, heads, kv_heads, dim, vdim, pag
     for s, (c, l) in enumerate(zip(ctx, lens)):
         last = row + l - 1
         special = 3 if window is None else c - window  # the last query's oldest visible key
+        if window is not None and special >= 1 and c > 2:
+            # the key just behind the last query's window would score half as much again: it must not show,
+            # for a single token no more than in a portion
+            keys[s][special - 1] = 1.5 * keys[s][special]
         if special >= 0 and c > 2:
             for h in range(heads):
                 k = keys[s][special, h // (heads // kv_heads)]
