@@ -4,7 +4,9 @@
 //   the `top` experts with the largest s + correction are chosen (the lowest index wins a tie);
 //   their weights are their s divided by the chosen experts' sum (+ 1e-20);
 //   out = sum over the chosen of weight * W_down_e (act(W_gate_e x) * (W_up_e x))  (+ what a
-//   shared expert gave).
+//   shared expert gave, times sigmoid of a number per token where the design gates it).
+//   Experts without a gate whose activation is the square of ReLU are the same with ReLU as act and
+//   their one matrix in both places: relu(u) * u; the kernels then form that product once.
 //
 // moe_route_kernel     a wavefront per token
 // moe_gate_up_kernel   a workgroup per (token, chosen expert, block of features): every
@@ -290,28 +292,28 @@ __global__ void __launch_bounds__(256)
                                                                  __builtin_bit_cast(mbf16x8, av[u][a]), accg[a][b], 0, 0, 0);
     }
   } else {
-  for (int k0 = 0; k0 < width; k0 += 32) {
-    const bool have = k0 + kg * 8 < width;  // (width is a multiple of 8: a piece is whole or absent)
-    uint4 av[2], gv[2], uv[2];
+    for (int k0 = 0; k0 < width; k0 += 32) {
+      const bool have = k0 + kg * 8 < width;  // (width is a multiple of 8: a piece is whole or absent)
+      uint4 av[2], gv[2], uv[2];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      av[a] = gv[a] = uv[a] = make_uint4(0, 0, 0, 0);
-      if (have) {
-        if (pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(xr[a] + k0);
-        gv[a] = *reinterpret_cast<const uint4*>(gr[a] + k0);
-        uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
+      for (int a = 0; a < 2; ++a) {
+        av[a] = gv[a] = uv[a] = make_uint4(0, 0, 0, 0);
+        if (have) {
+          if (pair[a] >= 0) av[a] = *reinterpret_cast<const uint4*>(xr[a] + k0);
+          gv[a] = *reinterpret_cast<const uint4*>(gr[a] + k0);
+          uv[a] = *reinterpret_cast<const uint4*>(ur[a] + k0);
+        }
       }
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, gv[b]),
+                                                               __builtin_bit_cast(mbf16x8, av[a]), accg[a][b], 0, 0, 0);
+          accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
+                                                               __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
+        }
     }
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, gv[b]),
-                                                             __builtin_bit_cast(mbf16x8, av[a]), accg[a][b], 0, 0, 0);
-        accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mbf16x8, uv[b]),
-                                                             __builtin_bit_cast(mbf16x8, av[a]), accu[a][b], 0, 0, 0);
-      }
-  }
   }
   // features were the rows of the products: this lane holds features f0 + 16 b + 4 kg + r of pair row a * 16 + i
 #pragma unroll
